@@ -346,6 +346,9 @@ def cmd_util(a):
             print(f"{name}: {', '.join(flags) or '-'}")
     elif a.util_cmd == "hf-scan":
         return _hf_scan(a)
+    elif a.util_cmd == "trace-run":
+        from .tools.trace_run import main as trace_main
+        return trace_main(a.rest)
     return 0
 
 
@@ -478,6 +481,8 @@ def main(argv=None):
     hs.add_argument("uris", nargs="*")
     hs.add_argument("--models-path")
     hs.add_argument("--galleries")
+    trc = usub.add_parser("trace-run", help="replay a trace of engine steps on a model directory and write logits")
+    trc.add_argument("rest", nargs=argparse.REMAINDER, help="--model DIR --dtype T --out DIR --max-tokens N")
     fd = sub.add_parser("federated", help="run the federated load-balancing proxy")
     fd.add_argument("--address", default=os.environ.get("LOCALAI_ADDRESS", "0.0.0.0:8080"))
     fd.add_argument("--p2ptoken")

@@ -28,8 +28,8 @@ from ..utils import roctx
 from ..utils.pinned import PinnedRing
 from ..models.llama import ForwardBatch, LlamaModel, Workspace
 from ..ops.sampling import SamplerBatch
-from .kv_cache import KVCache, make_block_manager
-from .scheduler import Scheduler, SchedulerOutput, needs_host_state
+from .kv_cache import KVCache, LatentCache, SlotPool, make_block_manager
+from .scheduler import ScheduledSeq, Scheduler, SchedulerOutput, needs_host_state
 from .sequence import Request, Sequence, Status, StepOutput
 
 log = logging.getLogger("localai_tfp_amd.engine")
@@ -116,6 +116,10 @@ class EngineConfig:
     # time every GEMM shape of the model over the compiled tile / split candidates at load (ops/autotune.py)
     gemm_autotune: bool = __import__("os").environ.get("MX_GEMM_TUNE", "1") != "0"
     n_draft: int = 0  # speculative decoding: draft tokens per step (needs a draft model; 0 = off)
+    # scheduler + step planner in libmxrt when it is built (False: the Python scheduler, which replay_step drives)
+    native_scheduler: bool = True
+    # logits rows a step may return beyond one per sequence (replay_step: logits at chosen prompt positions)
+    logits_rows: int = 0
     spec_max_batch: int = 32  # speculate only on decode batches up to this size (latency-bound regime)
 
 
@@ -369,6 +373,17 @@ class LLMEngine:
             c.block_size = c.max_model_len
             c.enable_prefix_cache = False
             draft = None
+        # latent-cache models (models/vosotar.py): a paged pool of per-token latents, addressed like K / V blocks, plus
+        # one state slot per live sequence (SlotPool) for rows carried between steps. A cached block does not hold
+        # that carried state, so blocks are not shared between requests; no drafts, no TP
+        self.latent = getattr(model, "cache_kind", "") == "latent"
+        self.state_slots = None
+        self._replay: dict = {}
+        if self.latent:
+            if tp is not None:
+                raise ValueError("tensor parallelism is not supported for latent-cache models")
+            c.enable_prefix_cache = False
+            draft = None
         self.max_blocks_per_seq = (c.max_model_len + c.block_size - 1) // c.block_size
         use_spec = draft is not None and c.n_draft > 0 and tp is None
         frac = c.kv_mem_fraction
@@ -385,6 +400,13 @@ class LLMEngine:
         if self.recurrent:
             nb = c.max_num_seqs + 1
             self.kv = model.make_state_cache(nb, c.block_size)
+        elif self.latent:
+            ranks = model.cache_ranks()
+            nb = c.num_blocks or LatentCache.auto_num_blocks(ranks, c.block_size, self.device, frac,
+                                                             dtype_bytes=model.dtype.itemsize)
+            self.kv = model.make_cache(nb, c.block_size, c.max_num_seqs)
+            self.state_slots = SlotPool(c.max_num_seqs)
+            self.cfg.use_graphs = False  # steps of this family launch eagerly
         else:
             nl = getattr(model, "kv_layers", mc.n_layers)
             nb = c.num_blocks or KVCache.auto_num_blocks(max(1, nl), model.n_kv, c.block_size, mc.head_dim,
@@ -400,13 +422,17 @@ class LLMEngine:
         # scheduler + step planner: native (csrc/runtime/scheduler.cpp) on the native block manager; the Python
         # Scheduler is the reference implementation (MX_PY_SCHED=1, or no libmxrt)
         from . import native_scheduler as NS
-        self.native_sched = (os.environ.get("MX_PY_SCHED", "0") != "1" and hasattr(self.bm, "_h") and NS.available())
+        self.native_sched = (c.native_scheduler and os.environ.get("MX_PY_SCHED", "0") != "1" and hasattr(self.bm, "_h")
+                             and NS.available())
         sched_cls = NS.NativeScheduler if self.native_sched else Scheduler
         self.sched = sched_cls(self.bm, c.block_size, c.max_num_seqs, c.max_batched_tokens, c.max_model_len,
                                prefill_chunk=c.prefill_chunk)
         max_parts = max(1, -(-c.max_model_len // c.attn_part_size))
         if self.recurrent:
             self.ws = model.make_workspace(max(c.max_batched_tokens, c.max_num_seqs), c.max_num_seqs)
+        elif self.latent:
+            self.ws = model.make_workspace(max(c.max_batched_tokens, c.max_num_seqs), c.max_num_seqs, c.logits_rows,
+                                           max_parts)
         else:
             # rows: a mixed step's graph bucket pads its decode rows to the decode bucket (<= max_num_seqs) and its
             # prompt tokens to the next mixed-graph token bucket, so the workspace holds both paddings at once
@@ -449,7 +475,8 @@ class LLMEngine:
         self.overlap = bool(c.overlap and not use_spec and not self.recurrent
                             and getattr(model, "remote", None) is None
                             and os.environ.get("MX_TP_OVERLAP", "1") != "0" if tp is not None else
-                            c.overlap and not use_spec and not self.recurrent and getattr(model, "remote", None) is None)
+                            c.overlap and not use_spec and not self.recurrent and not self.latent
+                            and getattr(model, "remote", None) is None)
         # rows whose next sample needs host state advanced by their in-flight token (a grammar mask, mirostat-2's
         # mu): by default they stay in every step — the step's forward is launched first and the previous step is
         # read while it runs, before the sampler (see _step_overlap). MX_OVERLAP_HOLD=1: such a row sits out
@@ -1051,6 +1078,12 @@ class LLMEngine:
         """The Python-side rest of a plan: multimodal spans, embedding rows, prefill attention tiles, graph bucket."""
         pf = so.prefill
         nd = plan["nd"]
+        if self.state_slots is not None:
+            # state slot of each sequence of the step (decode rows first). Slots of sequences that left the running
+            # set (finished, aborted, preempted) return to the pool first; a preempted one restarts at position 0
+            sp = self.state_slots
+            sp.keep_only({s.rid for s in self.sched.running})
+            plan["seq_state"] = np.asarray([sp.get(it.seq.rid) for it in list(so.decode) + list(pf)], np.int32)
         mm = []
         row = nd
         for it in pf:  # multimodal spans intersecting this chunk -> (row in T, embedding rows)
@@ -1090,7 +1123,7 @@ class LLMEngine:
                 logits = self.model.finish_logits(logits, self.ws)
             return logits, am
         t = self._stage_plan(plan, ("tokens", "positions", "slots", "lidx", "dec_bt", "dec_lens", "pf_bt", "pf_cu",
-                                    "pf_ctx", "pf_tseq", "pf_tq0"))
+                                    "pf_ctx", "pf_tseq", "pf_tq0", "seq_state"))
         fb = self._build_fb(plan, t)
         if "fix_dst" in t and fb.tokens.is_cuda:
             # one kernel (no int64 casts + index_select + index_copy launches)
@@ -1193,8 +1226,9 @@ class LLMEngine:
         nd = plan["nd"]
         if t is None:
             t = self._stage_plan(plan, ("tokens", "positions", "slots", "lidx", "dec_bt", "dec_lens", "pf_bt",
-                                        "pf_cu", "pf_ctx"))
+                                        "pf_cu", "pf_ctx", "seq_state"))
         fb = ForwardBatch(t["tokens"], t["positions"], t["slots"], t["lidx"], n_decode=nd)
+        fb.seq_state = t.get("seq_state")
         if nd:
             fb.dec_block_tables, fb.dec_seq_lens = t["dec_bt"], t["dec_lens"]
             fb.dec_max_len = int(plan["dec_lens"].max())
@@ -1383,6 +1417,68 @@ class LLMEngine:
             self.sched.finish(s, reason)
         s.finish_reason = reason
         self._emit(s, "", reason)
+
+    # ------------------------------------------------------------------ trace replay
+    def replay_step(self, entries, end=()):
+        """Run ONE engine step whose composition the caller dictates instead of the scheduler: `entries` is a list of
+        (key, next token ids, wanted positions among them) per request, all one batch. A request is admitted at its
+        first entry (a state slot, blocks as it grows); an entry of one token that continues a request is a decode
+        row, anything else a prompt chunk. Returns the fp32 logits [sum of wanted, vocab] in entry order (None if
+        nothing is wanted). `end` names the requests that are finished after the step: their blocks and slot return
+        to the pools. Sampling is not involved; block manager, planner, forward and kernels are the serving path's.
+        Needs the Python scheduler (EngineConfig.native_scheduler = False)."""
+        if self.native_sched or self.tp is not None:
+            raise RuntimeError("replay_step drives the Python scheduler of a single-rank engine")
+        so = SchedulerOutput()
+        items = []
+        for key, tokens, want in entries:
+            s = self._replay.get(key)
+            if s is None:
+                if len(self.sched.running) >= self.cfg.max_num_seqs:
+                    raise MemoryError("no free sequence slot")
+                s = Sequence(Request([], max_tokens=0, cache_prompt=False), self.tok)
+                s.status = Status.RUNNING
+                self.sched.running.append(s)
+                self._replay[key] = s
+            n, start = len(tokens), s.num_computed
+            if n == 0 or any(not 0 <= w < n for w in want):
+                raise ValueError("replay_step: an entry needs tokens, and wanted positions lie among them")
+            if start + n > self.cfg.max_model_len:
+                raise ValueError("replay_step: request longer than max_model_len")
+            s.prompt_ids.extend(int(x) for x in tokens)
+            if not self.sched._grow(s, start + n):
+                raise MemoryError("KV cache exhausted")
+            it = ScheduledSeq(s, start, n, False)
+            (so.decode if n == 1 and start > 0 else so.prefill).append(it)
+            items.append((it, want))
+        out = None
+        if not so.empty:
+            if so.num_tokens > self.ws.max_tokens:
+                raise ValueError(f"step of {so.num_tokens} tokens, engine built for {self.ws.max_tokens}")
+            plan = self._plan(so)
+            row0, r = {}, 0
+            for it in so.decode:
+                row0[id(it)] = r
+                r += 1
+            for it in so.prefill:
+                row0[id(it)] = r
+                r += it.n
+            plan["lidx"] = np.asarray([row0[id(it)] + w for it, want in items for w in want], np.int32)
+            plan["graph"] = False
+            logits, _ = self._execute(plan)
+            self.sched.commit(so)
+            self.stats["steps"] += 1
+            self.stats["decode_tokens"] += len(so.decode)
+            self.stats["prefill_tokens"] += sum(p.n for p in so.prefill)
+            if len(plan["lidx"]):
+                out = logits[:len(plan["lidx"])].float().cpu()
+        for key in end:
+            s = self._replay.pop(key, None)
+            if s is not None:
+                self.sched.finish(s, "stop")
+                if self.state_slots is not None:
+                    self.state_slots.release(s.rid)
+        return out
 
     # ------------------------------------------------------------------ convenience
     def generate(self, prompt_ids, params=None, max_tokens=32, stop=None) -> StepOutput:

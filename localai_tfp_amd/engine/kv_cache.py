@@ -165,3 +165,71 @@ def make_block_manager(num_blocks: int, block_size: int, enable_prefix_cache: bo
         return NativeBlockManager(num_blocks, block_size, enable_prefix_cache)
     except Exception:
         return PyBlockManager(num_blocks, block_size, enable_prefix_cache)
+
+
+class LatentCache:
+    """Cache of decoders that keep one low-rank latent per token and layer (ops/latent.py) plus a few carried input
+    rows per sequence and layer (the tails of a causal tap convolution):
+
+    * `lat[i]`: paged pool [num_blocks, block_size, rank_i] of layer i, bf16 or fp32, addressed by the same block
+      tables and flat slots (block * block_size + offset) as the K / V pools of `KVCache`;
+    * `tails[i]`: [num_state_slots, taps - 1, width] fp32, one slot per live sequence (`SlotPool`).
+
+    Ranks may differ between layers, so each layer owns its tensors."""
+
+    def __init__(self, ranks, num_blocks: int, block_size: int, device, dtype=torch.bfloat16, state_slots: int = 0,
+                 tail_rows: int = 0, width: int = 0):
+        self.n_layers, self.num_blocks, self.block_size = len(ranks), num_blocks, block_size
+        self.lat = [torch.zeros((num_blocks, block_size, int(r)), dtype=dtype, device=device) for r in ranks]
+        self.tails = [torch.zeros((max(1, state_slots), max(1, tail_rows), width), dtype=torch.float32, device=device)
+                      for _ in ranks]
+        self.state_slots = state_slots
+
+    def layer(self, i: int):
+        return self.lat[i], self.tails[i]
+
+    @staticmethod
+    def bytes_per_block(ranks, block_size: int, dtype_bytes: int = 2) -> int:
+        return int(sum(int(r) for r in ranks) * block_size * dtype_bytes)
+
+    @classmethod
+    def auto_num_blocks(cls, ranks, block_size: int, device, fraction: float = 0.85, reserve_bytes: int = 4 << 30,
+                        cap: int | None = None, dtype_bytes: int = 2) -> int:
+        dev = torch.device(device)
+        if dev.type != "cuda":
+            n = 4096
+        else:
+            free, _total = torch.cuda.mem_get_info(dev)
+            n = int(max(0, free * fraction - reserve_bytes) // max(1, cls.bytes_per_block(ranks, block_size, dtype_bytes)))
+        if cap:
+            n = min(n, cap)
+        return max(n, 16)
+
+
+class SlotPool:
+    """State slots of live sequences: a free list of `n` slots keyed by request id. A sequence takes a slot with
+    its first scheduled tokens and keeps it until it finishes, is aborted or is preempted (its state is then
+    recomputed from position 0 in whatever slot it gets next)."""
+
+    def __init__(self, n: int):
+        self.n = n
+        self.free = collections.deque(range(n))
+        self.owner: dict[int, int] = {}
+
+    def get(self, rid: int) -> int:
+        s = self.owner.get(rid)
+        if s is None:
+            if not self.free:
+                raise MemoryError("no free sequence-state slot")
+            s = self.owner[rid] = self.free.popleft()
+        return s
+
+    def release(self, rid: int) -> None:
+        s = self.owner.pop(rid, None)
+        if s is not None:
+            self.free.append(s)
+
+    def keep_only(self, rids) -> None:
+        """Release the slots of every owner not in `rids`."""
+        for r in [r for r in self.owner if r not in rids]:
+            self.release(r)

@@ -106,6 +106,7 @@ class ForwardBatch:
     tp_local_logits: bool = False  # tensor parallel: return this rank's vocabulary shard (no all-gather)
     stop_layer: int | None = None  # return the fp32 residual rows after this many layers (HF hidden_states[k])
     embed_rows: list | None = None  # [(row, fp32 [n, hidden])] input embeddings replacing token rows
+    seq_state: torch.Tensor | None = None  # int32 [n_decode + S_p] state slot of each sequence (latent-cache models)
 
     @property
     def T(self) -> int:

@@ -38,6 +38,9 @@ def load_llm(model: str, device="cpu", tp_rank: int = 0, tp_size: int = 1, tp_gr
     """-> (LlamaModel, tokenizer, LlamaConfig, metadata dict)"""
     from ..tokenizer import ByteTokenizer, from_gguf
     ov = overrides or {}
+    lat = _load_latent(model, device, tp_size, ov)
+    if lat is not None:
+        return lat
     rec = _load_recurrent(model, device, tp_size)
     if rec is not None:
         if ov.get("lora"):
@@ -143,6 +146,35 @@ def _apply_overrides(cfg: LlamaConfig, ov: dict):
         cfg.rms_eps = float(ov["rms_norm_eps"])
     if ov.get("context_size"):
         cfg.ctx_train = max(cfg.ctx_train, int(ov["context_size"])) if ov.get("extend_context") else cfg.ctx_train
+
+
+def _load_latent(model: str, device, tp_size: int, ov: dict):
+    """Latent-attention decoders (models/vosotar.py): a directory whose config.json names the Vosotar architecture,
+    or `synthetic:vosotar-*` random weights. `overrides["dtype"]`: torch.bfloat16 (default on GPU) | torch.float32.
+    None for everything else."""
+    from . import vosotar as VO
+    from ..tokenizer import ByteTokenizer
+    synth = model.startswith("synthetic:vosotar")
+    if not synth and not VO.is_vosotar_dir(model):
+        return None
+    if tp_size > 1:
+        raise ValueError("tensor parallelism is not supported for Vosotar models")
+    if ov.get("lora"):
+        raise NotImplementedError("LoRA adapters are not supported for Vosotar models")
+    if synth:
+        key = model.split(":", 1)[1]
+        cfg = VO.make_config(name=key, **VO.SYNTHETIC[key])
+        m = VO.VosotarModel.load(cfg, VO.synthetic_source(cfg, seed=1), device, ov.get("dtype"))
+        return m, ByteTokenizer(cfg.vocab), cfg, {}
+    cfg, get = VO.dir_source(model)
+    tok = ByteTokenizer(cfg.vocab)
+    if os.path.isfile(os.path.join(model, "tokenizer.json")):
+        try:
+            from ..tokenizer import from_hf_dir
+            tok = from_hf_dir(model)
+        except Exception as ex:
+            log.warning("no usable tokenizer in %s (%s); byte-level fallback", model, ex)
+    return VO.VosotarModel.load(cfg, get, device, ov.get("dtype")), tok, cfg, {}
 
 
 RECURRENT_ARCHS = {"mamba", "rwkv6"}

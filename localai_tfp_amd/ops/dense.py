@@ -62,6 +62,25 @@ class Dense:
         out.copy_(self(x))
         return out
 
+    def into(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """out (fp32, contiguous, preallocated) = x W^T + b: 16-bit operands with the fp32 accumulator written as is,
+        fp32 operands in plain fp32. No allocation, so a captured graph sees static addresses."""
+        if x.dtype == torch.float32:
+            if self.b32 is not None:
+                torch.addmm(self.b32, x, self.wt, out=out)
+            else:
+                torch.mm(x, self.wt, out=out)
+            return out
+        if _fp32_out_ok(x.dtype):
+            if self.b32 is not None:
+                out.copy_(self.b32.expand_as(out))
+                torch.addmm(out, x, self.wt, out_dtype=torch.float32, out=out)
+            else:
+                torch.mm(x, self.wt, out_dtype=torch.float32, out=out)
+            return out
+        out.copy_(self(x))
+        return out
+
     def acc(self, x: torch.Tensor, acc: torch.Tensor) -> torch.Tensor:
         """acc (fp32) += x W^T + b — the residual add fused as GEMM beta = 1."""
         if x.dtype != torch.float32 and _fp32_out_ok(x.dtype) and acc.is_contiguous():
