@@ -144,6 +144,18 @@ def build_kernels(verbose=False) -> Path:
     return _build_lib("libmxk.so", srcs, headers, HIPCC, cflags, ["-fPIC"], verbose)
 
 
+def build_latent(verbose=False) -> Path:
+    """libmxl.so: the kernels of the latent-attention decoders (csrc/kernels/latent/). A library of its own, so a
+    fresh checkout that serves only such a model compiles these two files and not the whole kernel set."""
+    kdir = CSRC / "kernels"
+    srcs = sorted((kdir / "latent").glob("*.hip"))
+    headers = sorted(kdir.glob("*.h"))
+    cflags = [f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17", "-ffp-contract=fast",
+              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-I", str(kdir), "-Wno-unused-result",
+              "-Wno-unknown-warning-option"]
+    return _build_lib("libmxl.so", srcs, headers, HIPCC, cflags, ["-fPIC"], verbose)
+
+
 def build_runtime(verbose=False) -> Path:
     rdir = CSRC / "runtime"
     srcs = sorted(rdir.glob("*.cpp"))
@@ -162,6 +174,7 @@ def build_all(verbose=False):
     if not shutil.which(HIPCC) and not Path(HIPCC).exists():
         raise RuntimeError(f"hipcc not found at {HIPCC}")
     k = build_kernels(verbose)
+    build_latent(verbose)
     r = build_runtime(verbose)
     return k, r
 

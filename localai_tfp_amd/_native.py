@@ -118,6 +118,28 @@ KERNEL_SIGS = {
     "mxk_conv_tile_auto": [I, I],
 }
 
+L = C.c_long
+# libmxl.so (csrc/kernels/latent/): kernels of the latent-attention decoders (ops/latent.py)
+LATENT_SIGS = {
+    # table, is16, V, tokens, g, eps, out, ldo, T, C, stream
+    "mxl_embed_norm": [P, I, I, P, P, F, P, I, I, I, P],
+    # x, ldx, rows, g, eps, out32, ld32, out16, ld16, M, C, stream
+    "mxl_scalar_norm": [P, I, P, P, F, P, I, P, I, I, I, P],
+    # x, ldx, y, ldy, gate_pre, ldg, g, eps, M, C, stream
+    "mxl_gated_norm_add": [P, I, P, I, P, I, P, F, I, I, P],
+    # u, ldu, out, ldo, is16, M, F, stream
+    "mxl_relu2": [P, I, P, I, I, I, I, P],
+    # h, ldh, w, taps, tails, state, positions, n_dec, pf_cu, n_pf, out, ldo, is16, T, C, stream
+    "mxl_tap_conv": [P, I, P, I, P, P, P, I, P, I, P, I, I, I, I, P],
+    # y, ldy, q_rank, rank, wq, wkv, eps, cq, ldcq, cq16, cache, cache16, slots, T, stream
+    "mxl_latent_norm_append": [P, I, I, I, P, P, F, P, I, I, P, I, P, I, P],
+    # qa, qs_t, qs_h, cache, is16, bs, R, bt, bt_stride, cu_q, ctx, n_seqs, n_rows, row_base, out, os_t, os_h, scale,
+    # H, parts, part_len, part_ml, part_o, stream
+    "mxl_latent_attn": [P, L, L, P, I, I, I, P, I, P, P, I, I, I, P, L, L, F, I, I, I, P, P, P],
+    # ov, gate_pre, ldg, out, ldo, is16, H, T, dv, stream
+    "mxl_head_gate_pack": [P, P, I, P, I, I, I, I, I, P],
+}
+
 HIP_ERRORS = {1: "hipErrorInvalidValue", 2: "hipErrorOutOfMemory", 98: "hipErrorInvalidDeviceFunction",
               209: "hipErrorNoBinaryForGpu", 700: "hipErrorIllegalAddress", 719: "hipErrorLaunchFailure"}
 
@@ -158,6 +180,38 @@ def kernels():
     return _kernels
 
 
+_latent = None
+
+
+def latent_kernels():
+    """Load libmxl.so (latent-attention decoder kernels), building it first when the tree has none (a fresh
+    checkout; the build takes seconds). Raises NativeError if it cannot be built or loaded."""
+    global _latent
+    if _latent is None:
+        with _lock:
+            if _latent is None:
+                ensure_built("latent")
+                lib = _load("libmxl.so")
+                for n, sig in LATENT_SIGS.items():
+                    fn = getattr(lib, n)
+                    fn.argtypes = sig
+                    fn.restype = C.c_int
+                _latent = lib
+    return _latent
+
+
+def ensure_built(group: str) -> None:
+    """Build a native library of the tree if it is not there yet (never rebuilds one that is)."""
+    name = {"latent": "libmxl.so"}[group]
+    if (_LIBDIR / name).exists():
+        return
+    from . import _build
+    try:
+        {"latent": _build.build_latent}[group]()
+    except Exception as ex:
+        raise NativeError(f"could not build {name}: {ex}") from ex
+
+
 def runtime():
     """Load libmxrt.so (host runtime: GGUF parser, block allocator, grammar, store)."""
     global _runtime
@@ -194,9 +248,10 @@ def ensure_act(dtype) -> None:
 
 
 def kcall(name: str, *args):
-    fn = getattr(kernels(), name, None)
+    lib = latent_kernels() if name.startswith("mxl_") else kernels()
+    fn = getattr(lib, name, None)
     if fn is None:
-        raise NativeError(f"{name} not exported by libmxk.so (stale build?)")
+        raise NativeError(f"{name} not exported by {lib._name} (stale build?)")
     rc = fn(*args)
     if rc != 0:
         raise NativeError(f"{name} failed: {HIP_ERRORS.get(rc, rc)} ({rc})")
@@ -218,7 +273,7 @@ def ptr(t) -> int | None:
 def loaded_library_paths():
     """Paths of the native libraries loaded into this process (for diagnostics / tests)."""
     out = []
-    for lib in (_kernels, _runtime):
+    for lib in (_kernels, _runtime, _latent):
         if lib is not None:
             out.append(lib._name)
     return out

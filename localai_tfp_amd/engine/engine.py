@@ -1471,7 +1471,7 @@ class LLMEngine:
             self.stats["decode_tokens"] += len(so.decode)
             self.stats["prefill_tokens"] += sum(p.n for p in so.prefill)
             if len(plan["lidx"]):
-                out = logits[:len(plan["lidx"])].float().cpu()
+                out = logits[:len(plan["lidx"])].to("cpu", torch.float32, copy=True)
         for key in end:
             s = self._replay.pop(key, None)
             if s is not None:

@@ -1,0 +1,365 @@
+"""Vosotar (latent attention + carried tap convolution) on the engine against the plain float64 oracle of
+tests/oracle_vosotar.py: every mechanism alone, whole prompts, token-by-token decoding, prompt portions down to two
+tokens, unequal batches, reuse of freed blocks and state slots, far keys and block / partition borders with peaked
+softmax weights, odd sizes, greedy generation through the scheduler, and the trace runner's command line.
+
+Each engine test runs on the CPU plumbing path (fp32) and, marked gpu, on the HIP kernels in fp32 and bf16."""
+import json
+import math
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle_vosotar as O
+from localai_tfp_amd.engine.engine import EngineConfig, LLMEngine
+from localai_tfp_amd.models import vosotar as VO
+from localai_tfp_amd.ops import latent as LA
+from localai_tfp_amd.ops.sampling import SamplingParams
+from localai_tfp_amd.tokenizer import ByteTokenizer
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GPU = pytest.param("cuda", marks=pytest.mark.gpu)
+DEVS = ["cpu", GPU]
+# (device, dtype name, tolerance relative to the largest |logit|)
+RUNS = [("cpu", "float32", 2e-4), pytest.param("cuda", "float32", 2e-4, marks=pytest.mark.gpu),
+        pytest.param("cuda", "bfloat16", 6e-2, marks=pytest.mark.gpu)]
+
+
+def build(device="cpu", dtype="float32", seed=0, **kw):
+    cfg = VO.make_config(**kw)
+    get = VO.synthetic_source(cfg, seed)
+    model = VO.VosotarModel.load(cfg, get, torch.device(device), getattr(torch, dtype))
+    return cfg, {k: get(k) for k in get.names}, model
+
+
+def engine(model, max_tokens=256, seqs=4, bs=16, native=False, blocks=None):
+    ec = EngineConfig(max_num_seqs=seqs, max_batched_tokens=max_tokens, max_model_len=max_tokens, block_size=bs,
+                      num_blocks=blocks or (-(-max_tokens // bs) * seqs + 1), use_graphs=False, overlap=False,
+                      native_scheduler=native, logits_rows=max_tokens, gemm_autotune=False)
+    return LLMEngine(model, ByteTokenizer(model.cfg.vocab), ec)
+
+
+def oracle(cfg, tensors, tokens):
+    return O.forward(cfg.to_json(), tensors, tokens).float()
+
+
+def close(got, want, tol):
+    err = (got.double() - want.double()).abs().max().item() / want.abs().max().item()
+    assert err < tol, err
+
+
+def run_cuts(eng, key, tokens, cuts):
+    """Feed `tokens` of one request in portions of the given sizes; all logits, in order."""
+    out, at = [], 0
+    for i, n in enumerate(cuts):
+        last = at + n == len(tokens)
+        out.append(eng.replay_step([(key, tokens[at:at + n], list(range(n)))], [key] if last else []))
+        at += n
+    assert at == len(tokens)
+    return torch.cat(out)
+
+
+def toks(n, vocab, seed=0):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+# ------------------------------------------------------------------------------------------------ mechanisms alone
+class _FB:
+    def __init__(self, n_dec, chunks, positions, state, dev, slots=None, dec_bt=None, dec_lens=None, pf_bt=None,
+                 pf_ctx=None):
+        i32 = dict(dtype=torch.int32, device=dev)
+        self.T = n_dec + sum(chunks)
+        self.n_decode = n_dec
+        self.pf_cu_q = torch.tensor(np.concatenate([[0], np.cumsum(chunks)]), **i32) if chunks else None
+        self.positions = torch.tensor(positions, **i32)
+        self.slots = torch.tensor(slots if slots is not None else [-1] * self.T, **i32)
+        self.seq_state = torch.tensor(state, **i32)
+        self.dec_block_tables = None if dec_bt is None else torch.tensor(dec_bt, **i32)
+        self.dec_seq_lens = None if dec_lens is None else torch.tensor(dec_lens, **i32)
+        self.pf_block_tables = None if pf_bt is None else torch.tensor(pf_bt, **i32)
+        self.pf_ctx_lens = None if pf_ctx is None else torch.tensor(pf_ctx, **i32)
+        self.dec_max_len = max(dec_lens) if dec_lens else 0
+
+
+@pytest.mark.parametrize("dev", DEVS)
+def test_norms_gate_and_activation(dev):
+    g = torch.Generator().manual_seed(1)
+    M, C, eps = 5, 72, 0.3  # a large eps shows whether it sits inside the root
+    x = torch.randn(M, C, generator=g) * 3
+    gain = torch.tensor([1.7])
+    want = O.scalar_norm(x.double(), gain, eps)
+    o32 = torch.empty(M, C, device=dev)
+    o16 = torch.empty(M, C, device=dev, dtype=torch.bfloat16)
+    LA.scalar_rmsnorm(x.to(dev), gain.to(dev), eps, out32=o32, out16=o16)
+    close(o32.cpu(), want, 1e-5)
+    close(o16.float().cpu(), want, 1e-2)
+    rows = torch.tensor([3, 0, 3], dtype=torch.int32)
+    sel = torch.empty(3, C, device=dev)
+    LA.scalar_rmsnorm(x.to(dev), gain.to(dev), eps, out32=sel, rows=rows.to(dev))
+    close(sel.cpu(), want[rows.long()], 1e-5)
+    # embedding gather + norm
+    table = torch.randn(11, C, generator=g).to(torch.bfloat16)
+    ids = torch.tensor([10, 0, 4, 4], dtype=torch.int32)
+    e = torch.empty(4, C, device=dev)
+    LA.embed_scalar_norm(table.to(dev), ids.to(dev), gain.to(dev), eps, e)
+    close(e.cpu(), O.scalar_norm(table.double()[ids.long()], gain, eps), 1e-5)
+    # x += gain * unit_rms(y * sigmoid(gate)); the gate is a column slice of a wider buffer
+    y, wide = torch.randn(M, C, generator=g), torch.randn(M, C + 9, generator=g)
+    res = x.clone().to(dev)
+    LA.gated_norm_add(res, y.to(dev), wide.to(dev)[:, 9:], gain.to(dev), eps)
+    close(res.cpu(), x.double() + O.scalar_norm(y.double() * torch.sigmoid(wide.double()[:, 9:]), gain, eps), 1e-5)
+    # squared relu on a column slice
+    a = torch.empty(M, C, device=dev)
+    LA.relu2(wide.to(dev)[:, :C], a)
+    close(a.cpu(), torch.relu(wide.double()[:, :C]) ** 2, 1e-6)
+    # per-head output gate + pack
+    H, dv = 3, 5
+    ov, gp = torch.randn(H, M, dv, generator=g), torch.randn(M, H + 2, generator=g)
+    pk = torch.empty(M, H * dv, device=dev)
+    LA.head_gate_pack(ov.to(dev), gp.to(dev)[:, 2:], pk)
+    close(pk.cpu(), (ov.double().permute(1, 0, 2) * torch.sigmoid(gp.double()[:, 2:, None])).reshape(M, H * dv), 1e-6)
+
+
+@pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("taps", [1, 2, 3, 5])
+def test_tap_conv_carries_tails_across_steps(dev, taps):
+    g = torch.Generator().manual_seed(taps)
+    C, n = 70, 23
+    w = torch.randn(C, taps, generator=g)
+    seqs = [torch.randn(n, C, generator=g) for _ in range(3)]
+    want = [s.double() + O.tap_conv(s.double(), w) for s in seqs]
+    tails = torch.full((4, max(1, taps - 1), C), 7.0, device=dev)  # stale contents must not leak into a new sequence
+    slot = [2, 0, 3]
+    # sequence 0: portions 1, 2, 1 (decode row), 6, 13; sequence 1: whole, one step late; sequence 2: token by token
+    plan = {0: [1, 2, 1, 6, 13], 1: [0, 23], 2: [1] * 23}
+    at = [0, 0, 0]
+    got = [torch.zeros(n, C) for _ in range(3)]
+    for step in range(23):
+        dec, chunks = [], []
+        for s in range(3):
+            k = plan[s][step] if step < len(plan[s]) else 0
+            if k:
+                (dec if k == 1 and at[s] > 0 else chunks).append((s, k))
+        order = dec + chunks
+        if not order:
+            continue
+        h = torch.cat([seqs[s][at[s]:at[s] + k] for s, k in order])
+        pos = [p for s, k in order for p in range(at[s], at[s] + k)]
+        fb = _FB(len(dec), [k for _, k in chunks], pos, [slot[s] for s, _ in order], dev)
+        out = torch.empty(h.shape, device=dev)
+        LA.tap_conv(h.to(dev), w.to(dev), tails, LA.Ragged(fb), out)
+        r = 0
+        for s, k in order:
+            got[s][at[s]:at[s] + k] = out[r:r + k].cpu()
+            r += k
+            at[s] += k
+    for s in range(3):
+        close(got[s], want[s], 1e-5)
+
+
+@pytest.mark.parametrize("dev,dt", [("cpu", "float32"), pytest.param("cuda", "float32", marks=pytest.mark.gpu),
+                                    pytest.param("cuda", "bfloat16", marks=pytest.mark.gpu)])
+@pytest.mark.parametrize("R,H", [(40, 3), (64, 8), (130, 2), (300, 1)])
+def test_latent_attention_far_keys_and_borders(dev, dt, R, H):
+    """Absorbed attention over paged latents: one planted key per query carries nearly all the weight, placed far
+    back, at a block's last / first slot, at the newest position, and (decode) across the partition length."""
+    g = torch.Generator().manual_seed(R)
+    dtype = getattr(torch, dt)
+    bs, ctx, nblk = 16, 700, 64
+    lat = torch.randn(ctx, R, generator=g)
+    lat = (lat / lat.norm(dim=-1, keepdim=True)).to(dtype).float()
+    perm = torch.randperm(nblk - 1, generator=g)[:-(-ctx // bs)] + 1
+    cache = torch.zeros(nblk, bs, R)
+    cache.view(-1, R)[(perm.repeat_interleave(bs)[:ctx] * bs + torch.arange(ctx) % bs)] = lat
+    scale = 0.5
+
+    def planted(pos_keys):
+        """queries (H rows each) that point at the given keys with weight ~1"""
+        q = torch.randn(H, len(pos_keys), R, generator=g) * 0.1
+        for i, k in enumerate(pos_keys):
+            q[:, i] += 40.0 * lat[k]
+        return q.to(dtype)
+
+    def want(q, positions):
+        s = torch.einsum("hnr,jr->hnj", q.double(), lat.double()) * scale
+        vis = torch.arange(ctx)[None, :] <= torch.tensor(positions)[:, None]
+        return torch.einsum("hnj,jr->hnr", torch.softmax(s.masked_fill(~vis[None], -math.inf), -1), lat.double())
+
+    # a chunk of the last 37 rows (ctx 700) beside two decode rows of other lengths
+    n = 37
+    chunk_pos = list(range(ctx - n, ctx))
+    keys = [0, 15, 16, 511, 512, 3, ctx - n - 1, ctx - n] + [p for p in chunk_pos[8:]]  # the tail points at itself
+    dec_lens = [530, 17]
+    dec_keys = [5, 16]
+    q = torch.cat([planted(dec_keys), planted(keys)], 1)
+    bt = perm.tolist()
+    fb = _FB(2, [n], [l - 1 for l in dec_lens] + chunk_pos, [0, 1, 2], dev, dec_bt=[bt, bt], dec_lens=dec_lens,
+             pf_bt=[bt], pf_ctx=[ctx])
+    out = torch.empty(H, 2 + n, R, device=dev, dtype=dtype)
+    ws = (torch.empty(2 * H * 8, 2, device=dev), torch.empty(2 * H * 8, R, device=dev))
+    LA.latent_attention(q.to(dev), cache.to(dev).to(dtype), LA.Ragged(fb), scale, out, workspace=ws, part_len=128)
+    ref = want(q.float(), [l - 1 for l in dec_lens] + chunk_pos)
+    close(out.float().cpu(), ref, 1e-4 if dt == "float32" else 2e-2)
+    # the planted keys really dominate: a kernel that skipped them would be far off
+    assert (ref[:, 2, :] - lat[0].double()).abs().max() < 0.05
+
+
+# ------------------------------------------------------------------------------------------------ whole model
+SHAPES = {
+    "plain": dict(hidden=64, vocab=97, n_layers=2, heads=4, dim=16, vdim=16, kv_rank=32, q_rank=48, ff=96),
+    # one head, key and value sizes that differ, a rank that is no multiple of 32, width no multiple of 64,
+    # two taps, borrowed layers, a large eps and a scale that is not dim^-1/2
+    "odd": dict(hidden=72, vocab=61, n_layers=2, heads=1, dim=24, vdim=40, kv_rank=40, q_rank=20, ff=50, taps=2,
+                shared=3, eps=0.05, scale=0.9),
+    "wide_rank": dict(hidden=48, vocab=50, n_layers=1, heads=5, dim=8, vdim=12, kv_rank=136, q_rank=8, ff=64, taps=4,
+                      shared=1, scale=1.5),
+    "one_tap": dict(hidden=64, vocab=40, n_layers=2, heads=2, dim=32, vdim=8, kv_rank=16, q_rank=64, ff=32, taps=1),
+}
+
+
+def no_ff(cfg):
+    cfg.layers[-1].ff = None
+    return cfg
+
+
+@pytest.mark.parametrize("dev,dt,tol", RUNS)
+@pytest.mark.parametrize("shape", list(SHAPES))
+def test_whole_prompt_decode_and_portions(dev, dt, tol, shape):
+    cfg, tensors, model = build(dev, dt, seed=3, **SHAPES[shape])
+    t = toks(75, cfg.vocab, 5)
+    want = oracle(cfg, tensors, t)
+    eng = engine(model, max_tokens=96, blocks=2 * 6 + 1)  # room for two requests: every run reuses freed blocks
+    close(run_cuts(eng, "w", t, [75]), want, tol)
+    close(run_cuts(eng, "d", t, [43] + [1] * 32), want, tol)
+    close(run_cuts(eng, "c", t, [2, 3, 1, 16, 2, 15, 9, 17, 2, 1, 1, 2, 4]), want, tol)
+    close(run_cuts(eng, "t", t[:40], [1] * 40), want[:40], tol)
+
+
+@pytest.mark.parametrize("dev,dt,tol", RUNS)
+def test_layer_without_feed_forward(dev, dt, tol):
+    cfg = no_ff(VO.make_config(**SHAPES["plain"]))
+    get = VO.synthetic_source(cfg, 9)
+    model = VO.VosotarModel.load(cfg, get, torch.device(dev), getattr(torch, dt))
+    assert not any(n.startswith("l1.mlp") or n.startswith("l1.rg2") or n.startswith("l1.norm2") for n in get.names)
+    t = toks(30, cfg.vocab, 2)
+    close(run_cuts(engine(model, 64), "a", t, [7, 1, 22]), oracle(cfg, {k: get(k) for k in get.names}, t), tol)
+
+
+@pytest.mark.parametrize("dev,dt,tol", RUNS)
+def test_mixed_batches_and_reused_blocks_and_slots(dev, dt, tol):
+    """Up to three live requests of unequal length in one step (portions beside single tokens), in a pool of two
+    state slots less than the requests and blocks that must be used again; each equals the request run alone."""
+    cfg, tensors, model = build(dev, dt, seed=11, **SHAPES["odd"])
+    reqs = {k: toks(n, cfg.vocab, i) for i, (k, n) in enumerate([("a", 50), ("b", 33), ("c", 64), ("d", 18), ("e", 41)])}
+    want = {k: oracle(cfg, tensors, v) for k, v in reqs.items()}
+    eng = engine(model, max_tokens=96, seqs=3, blocks=3 * 4 + 1 + 1)
+    plan = [[("a", 20)], [("a", 1), ("b", 31)], [("a", 1), ("b", 1), ("c", 2)], [("c", 30), ("b", 1), ("a", 28)],
+            [("c", 1)], [("d", 18), ("c", 31)], [("e", 2)], [("e", 1), ("d", 0)], [("e", 38)]]
+    got = {k: [] for k in reqs}
+    at = {k: 0 for k in reqs}
+    for step in plan:
+        entries, end = [], []
+        for k, n in step:
+            if n == 0:
+                continue
+            entries.append((k, reqs[k][at[k]:at[k] + n], list(range(n))))
+            at[k] += n
+            if at[k] == len(reqs[k]):
+                end.append(k)
+        out = eng.replay_step(entries, end)
+        r = 0
+        for k, tk, _ in entries:
+            got[k].append(out[r:r + len(tk)])
+            r += len(tk)
+    for k in reqs:
+        assert at[k] == len(reqs[k])
+        close(torch.cat(got[k]), want[k], tol)
+    assert eng.bm.num_free == eng.bm.num_blocks - 1 and len(eng.state_slots.free) == 3
+
+
+@pytest.mark.parametrize("dev,dt,tol", RUNS)
+def test_peaked_attention_long_context_and_long_decode(dev, dt, tol):
+    """A large softmax scale makes single keys dominate, so a lost or shifted key anywhere in 600 tokens of context
+    (block borders, the decode partition length) moves the logits; then 90 tokens decoded one by one."""
+    kw = dict(SHAPES["plain"], scale=3.0, n_layers=1, shared=1)
+    cfg, tensors, model = build(dev, dt, seed=21, **kw)
+    t = toks(690, cfg.vocab, 8)
+    want = oracle(cfg, tensors, t)
+    eng = engine(model, max_tokens=704, seqs=2)
+    got = run_cuts(eng, "x", t, [509, 3, 88] + [1] * 90)
+    close(got, want, tol * 2)
+
+
+# ------------------------------------------------------------------------------------------------ serving path
+@pytest.mark.parametrize("dev,dt", [("cpu", "float32"), pytest.param("cuda", "float32", marks=pytest.mark.gpu)])
+@pytest.mark.parametrize("native", [False, True])
+def test_greedy_generation_through_the_scheduler(dev, dt, native):
+    """engine.generate / submit: chunked prefill, continuous batching of three requests, greedy sampling; each
+    request's tokens equal the oracle's greedy continuation."""
+    cfg, tensors, model = build(dev, dt, seed=4, **SHAPES["plain"])
+    ec = EngineConfig(max_num_seqs=2, max_batched_tokens=24, prefill_chunk=10, max_model_len=128, block_size=16,
+                      num_blocks=20, use_graphs=False, native_scheduler=native, gemm_autotune=False)
+    eng = LLMEngine(model, ByteTokenizer(cfg.vocab), ec)
+    if native and not eng.native_sched:
+        pytest.skip("native runtime not built")
+    prompts = [toks(n, cfg.vocab, 30 + n) for n in (27, 5, 13)]
+    from localai_tfp_amd.engine.sequence import Request
+    hs = [eng.submit(Request(p, SamplingParams(temperature=0.0, ignore_eos=True), 12)) for p in prompts]
+    eng.run_until_done()
+    for p, h in zip(prompts, hs):
+        ids = [i for o in h for i in o.token_ids]
+        seq = list(p)
+        for _ in range(12):
+            seq.append(int(oracle(cfg, tensors, seq)[-1].argmax()))
+        assert ids == seq[len(p):]
+    assert len(eng.state_slots.owner) <= 2
+
+
+def test_config_reader_and_checkpoint_round_trip(tmp_path):
+    cfg = VO.make_config(**SHAPES["odd"])
+    cfg.layers[1].ff = cfg.layers[3].ff = None  # layer 3 borrows layer 1's tensors
+    get = VO.synthetic_source(cfg, 1)
+    VO.save_checkpoint(cfg, get, str(tmp_path))
+    assert VO.is_vosotar_dir(str(tmp_path))
+    cfg2, get2 = VO.dir_source(str(tmp_path))
+    assert cfg2.to_json() == cfg.to_json() and cfg2.layers[2].weights_of == 0 and cfg2.layers[1].ff is None
+    assert torch.equal(get2("l1.mix.uk"), get("l1.mix.uk")) and get2("l2.mix.uk") is None
+    from localai_tfp_amd.models.loader import load_llm
+    m, _tok, c, _ = load_llm(str(tmp_path), "cpu")
+    assert isinstance(m, VO.VosotarModel) and c.taps == 2
+    bad = cfg.to_json()
+    bad["layers"][0]["type"] = "something_else"
+    with pytest.raises(ValueError):
+        VO.VosotarConfig.from_json(bad)
+    bad = cfg.to_json()
+    bad["layers"][0]["mlp"]["kind"] = "sparse"
+    with pytest.raises(ValueError):
+        VO.VosotarConfig.from_json(bad)
+
+
+def test_trace_runner_command_line(tmp_path):
+    """bin/trace_run on a checkpoint directory: steps on stdin, one logits file per step that wants any."""
+    cfg = VO.make_config(**SHAPES["wide_rank"])
+    get = VO.synthetic_source(cfg, 6)
+    mdir, odir = str(tmp_path / "m"), str(tmp_path / "o")
+    VO.save_checkpoint(cfg, get, mdir)
+    a, b = toks(21, cfg.vocab, 1), toks(9, cfg.vocab, 2)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:12], "want": [0, 11]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[12:13], "want": []}, {"id": "b", "tokens": b, "want": [8]}],
+              "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[13:], "want": [7, 0]}], "end": ["a"]}]
+    r = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", mdir, "--dtype", "float32", "--out", odir,
+                        "--max-tokens", "128", "--device", "cpu"], input="".join(json.dumps(s) + "\n" for s in steps),
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [ln for ln in r.stdout.splitlines() if ln.startswith("done")] == ["done 0", "done 1", "done 2"]
+    tensors = {k: get(k) for k in get.names}
+    wa, wb = oracle(cfg, tensors, a), oracle(cfg, tensors, b)
+    rd = lambda n: torch.from_numpy(np.fromfile(os.path.join(odir, "%d.f32" % n), dtype="<f4").reshape(-1, cfg.vocab))  # noqa: E731
+    close(rd(0), wa[[0, 11]], 2e-4)
+    close(rd(1), wb[[8]], 2e-4)
+    close(rd(2), wa[[20, 13]], 2e-4)
