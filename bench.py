@@ -96,6 +96,11 @@ def parse():
                     help="comma list of sampling phases measured back to back on the same server: reference = "
                          "the reference's defaults (temperature 0.9, top_k 40, top_p 0.95; backend_config.go "
                          "SetDefaults) on the GPU sampler; greedy = argmax. The first phase is the headline")
+    ap.add_argument("--arch-bench", default="", choices=["", "vosotar"],
+                    help="instead of the headline serving benchmark: prefill and decode throughput of this model "
+                         "family beside the Llama graph at equal layer sizes (random bf16 / f16 weights, one GPU)")
+    ap.add_argument("--arch-sizes", default="1b,7b", help="--arch-bench: comma list of layer sizes (1b, 7b)")
+    ap.add_argument("--arch-layers", type=int, default=4, help="--arch-bench: layers per model")
     return ap.parse_args()
 
 
@@ -203,8 +208,79 @@ def spawn_ranks(args) -> int | None:
     return p.returncode
 
 
+ARCH_SIZES = {"1b": dict(hidden=2048, heads=16, ff=8192, q_rank=768), "7b": dict(hidden=4096, heads=32, ff=14336, q_rank=1536)}
+
+
+def run_arch_bench(args) -> int:
+    """Prefill tokens/s (one prompt of P tokens per step) and decode tokens/s (B sequences at ~P tokens of context)
+    through the serving engine, greedy: the named family and the Llama graph with the same width, heads, head size,
+    feed-forward width, layer count and vocabulary. One JSON line per (size, model) and a summary line."""
+    import torch
+    from localai_tfp_amd.engine.engine import EngineConfig, LLMEngine
+    from localai_tfp_amd.engine.sequence import Request
+    from localai_tfp_amd.models import vosotar as VO
+    from localai_tfp_amd.models.config import LlamaConfig
+    from localai_tfp_amd.models.llama import LlamaModel
+    from localai_tfp_amd.models.synthetic import synthetic_source
+    from localai_tfp_amd.ops.sampling import SamplingParams
+    from localai_tfp_amd.tokenizer import ByteTokenizer
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    P, G, V, nl = args.prompt_len * 4, 64, 32000, args.arch_layers
+    rows = []
+
+    def models(sz):
+        s = ARCH_SIZES[sz]
+        vc = VO.make_config(hidden=s["hidden"], vocab=V, n_layers=nl, heads=s["heads"], dim=128, vdim=128, kv_rank=512,
+                            q_rank=s["q_rank"], ff=s["ff"], name=f"vosotar-{sz}")
+        yield "vosotar", lambda: VO.VosotarModel.load(vc, VO.synthetic_source(vc, 1), dev, torch.bfloat16)
+        lc = LlamaConfig(name=f"llama-{sz}", n_layers=nl, hidden=s["hidden"], ffn=s["ff"], n_heads=s["heads"],
+                         n_kv_heads=max(1, s["heads"] // 4), head_dim=128, vocab=V, ctx_train=8192, rope_base=10000.0,
+                         rope_dim=128)
+        yield "llama-f16", lambda: LlamaModel.load(lc, synthetic_source(lc, "F16", seed=1), dev)
+
+    def timed(eng, prompts, gen):
+        hs = [eng.submit(Request(list(p), SamplingParams(temperature=0.0, ignore_eos=True), gen)) for p in prompts]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.run_until_done()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert all(sum(len(o.token_ids) for o in h) == gen for h in hs)
+        return dt
+
+    rng = np.random.default_rng(0)
+    for sz in [x for x in args.arch_sizes.split(",") if x]:
+        for name, make in models(sz):
+            model = make()
+            for B in (1, 32):
+                ec = EngineConfig(max_num_seqs=B, max_batched_tokens=P, max_model_len=P + G + 64, block_size=16,
+                                  num_blocks=(B * (P + G + 64)) // 16 + 64, enable_prefix_cache=False,
+                                  use_graphs=not args.no_graphs)
+                eng = LLMEngine(model, ByteTokenizer(V), ec)
+                prompts = [rng.integers(0, V, P).tolist() for _ in range(B)]
+                timed(eng, prompts[:1], 2)  # warm-up: allocations, graph capture of the first bucket
+                timed(eng, prompts, G + 1)
+                reps = max(1, args.steps // 10)
+                t_p = min(timed(eng, prompts, 1) for _ in range(reps))
+                t_all = min(timed(eng, prompts, G + 1) for _ in range(reps))
+                r = {"size": sz, "model": name, "layers": nl, "batch": B, "prompt_len": P, "gen_len": G,
+                     "prefill_tok_s": round(B * P / t_p, 1), "decode_tok_s": round(B * G / max(t_all - t_p, 1e-9), 1),
+                     "weight_mb": round(model.weight_bytes() / 2 ** 20, 1), "graph_steps": eng.stats["graph_steps"]}
+                rows.append(r)
+                print(json.dumps(r), flush=True)
+                del eng
+            del model
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "arch_bench", "family": args.arch_bench, "unit": "tokens/s", "n_gpus": 1,
+                      "dtype": "bf16", "data": "synthetic", "rows": rows}), flush=True)
+    return 0
+
+
 def main():
     args = parse()
+    if args.arch_bench:
+        sys.exit(run_arch_bench(args))
     rc = spawn_ranks(args)
     if rc is not None:
         sys.exit(rc)

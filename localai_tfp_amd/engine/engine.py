@@ -219,6 +219,8 @@ class StepGraph:
         # (still unread) step scatters into it for the rows that need no fix
         lay = [("tokens", (T + 1,)), ("positions", (T,)), ("slots", (T,)), ("lidx", (self.S,)),
                ("dec_bt", (Bp, mb)), ("dec_lens", (Bp,)), ("fix_dst", (Bp,)), ("fix_src", (Bp,)), ("argmax_on", (1,))]
+        if e.state_slots is not None:  # state slot of each decode row (padded rows: -1, no state read or written)
+            lay += [("seq_state", (Bp,))]
         if P:
             lay += [("pf_bt", (PS, mb)), ("pf_cu", (PS + 1,)), ("pf_ctx", (PS,)), ("pf_tseq", (self.NT,)),
                     ("pf_tq0", (self.NT,))]
@@ -229,7 +231,8 @@ class StepGraph:
         self.n = o
         img = np.zeros(o, np.int32)
         self._default = img
-        for k, v in (("slots", -1), ("dec_lens", 1), ("pf_tseq", -1), ("fix_dst", T), ("argmax_on", 1)):
+        for k, v in (("slots", -1), ("dec_lens", 1), ("pf_tseq", -1), ("fix_dst", T), ("argmax_on", 1),
+                     ("seq_state", -1)):
             if k in self.off:
                 self.view(img, k)[...] = v
         self.buf = torch.from_numpy(img.copy()).to(dev)
@@ -242,6 +245,8 @@ class StepGraph:
         self.fb = ForwardBatch(v["tokens"][:T], v["positions"], v["slots"], v["lidx"], n_decode=B,
                                dec_block_tables=v["dec_bt"][:B], dec_seq_lens=v["dec_lens"][:B],
                                dec_max_len=L or e.cfg.max_model_len)
+        if "seq_state" in v:
+            self.fb.seq_state = v["seq_state"][:B] if B else v["seq_state"][:0]
         if P:
             self.fb.pf_block_tables, self.fb.pf_cu_q, self.fb.pf_ctx_lens = v["pf_bt"], v["pf_cu"], v["pf_ctx"]
             self.fb.pf_tiles = (v["pf_tseq"], v["pf_tq0"])
@@ -318,6 +323,8 @@ class StepGraph:
             bt = plan["dec_bt"]
             self.view(img, "dec_bt")[:nd, :bt.shape[1]] = bt
             self.view(img, "dec_lens")[:nd] = plan["dec_lens"]
+            if "seq_state" in self.off:
+                self.view(img, "seq_state")[:nd] = plan["seq_state"][:nd]
         if "pf_cu" in plan:
             bt, cu = plan["pf_bt"], plan["pf_cu"]
             ns = len(cu) - 1
@@ -406,7 +413,6 @@ class LLMEngine:
                                                              dtype_bytes=model.dtype.itemsize)
             self.kv = model.make_cache(nb, c.block_size, c.max_num_seqs)
             self.state_slots = SlotPool(c.max_num_seqs)
-            self.cfg.use_graphs = False  # steps of this family launch eagerly
         else:
             nl = getattr(model, "kv_layers", mc.n_layers)
             nb = c.num_blocks or KVCache.auto_num_blocks(max(1, nl), model.n_kv, c.block_size, mc.head_dim,

@@ -323,6 +323,28 @@ def test_greedy_generation_through_the_scheduler(dev, dt, native):
     assert len(eng.state_slots.owner) <= 2
 
 
+@pytest.mark.gpu
+def test_decode_graphs_replay_like_the_oracle():
+    """Decode-only steps replay captured graphs (several buckets as requests come and go, eager prompt chunks
+    between the replays); every request still yields the oracle's greedy tokens, also after slots were reused."""
+    cfg, tensors, model = build("cuda", "float32", seed=4, **SHAPES["odd"])
+    ec = EngineConfig(max_num_seqs=3, max_batched_tokens=32, prefill_chunk=9, max_model_len=128, block_size=16,
+                      num_blocks=24, use_graphs=True, gemm_autotune=False)
+    eng = LLMEngine(model, ByteTokenizer(cfg.vocab), ec)
+    from localai_tfp_amd.engine.sequence import Request
+    prompts = [toks(n, cfg.vocab, 70 + n) for n in (21, 4, 30, 11, 17)]
+    gens = [14, 25, 6, 9, 12]
+    hs = [eng.submit(Request(p, SamplingParams(temperature=0.0, ignore_eos=True), g)) for p, g in zip(prompts, gens)]
+    eng.run_until_done()
+    assert eng.stats["graph_steps"] > 10
+    for p, g, h in zip(prompts, gens, hs):
+        ids = [i for o in h for i in o.token_ids]
+        seq = list(p)
+        for _ in range(g):
+            seq.append(int(oracle(cfg, tensors, seq)[-1].argmax()))
+        assert ids == seq[len(p):]
+
+
 def test_config_reader_and_checkpoint_round_trip(tmp_path):
     cfg = VO.make_config(**SHAPES["odd"])
     cfg.layers[1].ff = cfg.layers[3].ff = None  # layer 3 borrows layer 1's tensors
