@@ -257,23 +257,282 @@ int dispatch(const AttnArgs& a, int n_rows, hipStream_t st) {
     return (int)hipErrorInvalidValue;
 }
 
+// ---- the same attention on the matrix cores (bf16 storage, R a multiple of 8) ----------------------------------
+// A workgroup of NW waves owns 16 NW consecutive (token, head) rows of one sequence; wave w holds rows 16 w .. + 15
+// as MFMA 16x16x32 A fragments (absorbed queries, read once from HBM into registers). The visible keys stream in
+// tiles of 32 latents through ONE LDS image [32][R_pad] shared by the waves, and the image serves both products:
+//   S = qa . c^T : B fragment = 8 consecutive rank entries of one key  -> a 16-byte ds_read of the key's row;
+//   O += P c     : B fragment = one rank entry of 8 consecutive keys   -> ds_read_b64_tr_b16, the hardware transpose
+//                  (a 16-lane group reads a 4-key x 16-entry block, lane l gets entry l of the 4 keys).
+// Scores, the online softmax and both accumulators are fp32; the weights are rounded to bf16 as MFMA operands.
+MX_DEV float group_max16(float v) {
+    v = fmaxf(v, __shfl_xor(v, 1, 64));
+    v = fmaxf(v, __shfl_xor(v, 2, 64));
+    v = fmaxf(v, __shfl_xor(v, 4, 64));
+    return fmaxf(v, __shfl_xor(v, 8, 64));
+}
+MX_DEV float group_sum16(float v) {
+    v += __shfl_xor(v, 1, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 4, 64);
+    return v + __shfl_xor(v, 8, 64);
+}
+
+template <int RV, int NW>
+__global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
+    constexpr int RP = RV * 32, KT = 32, CSTR = RP * 2 + 16, PSTR = KT * 2 + 16, BM = NW * 16, NTH = NW * 64;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    char* c_lds = smem;                                   // [KT][CSTR] bf16 latents of the tile
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, g = lane >> 4;
+    char* pw = smem + KT * CSTR + wave * 16 * PSTR;       // this wave's P [16][PSTR]
+    const int H = a.H, R = a.R;
+    const bf16_t* qa = (const bf16_t*)a.qa;
+    const bf16_t* cache = (const bf16_t*)a.cache;
+
+    int seq = -1, g0 = 0, qlen = 1, crow0 = 0;
+    {
+        int tile = blockIdx.x;
+        if (a.cu_q == nullptr) {
+            const int tps = (H + BM - 1) / BM;
+            seq = tile / tps;
+            g0 = (tile - seq * tps) * BM;
+            crow0 = seq;
+            if (seq >= a.n_seqs) return;
+        } else {
+            for (int s = 0; s < a.n_seqs; ++s) {
+                const int q = a.cu_q[s + 1] - a.cu_q[s];
+                const int nt = (q * H + BM - 1) / BM;
+                if (tile < nt) {
+                    seq = s;
+                    g0 = tile * BM;
+                    qlen = q;
+                    crow0 = a.cu_q[s];
+                    break;
+                }
+                tile -= nt;
+            }
+            if (seq < 0) return;
+        }
+    }
+    const int ctx = a.ctx[seq];
+    const int nrows = qlen * H;
+    const int t_last = min(qlen - 1, (g0 + BM - 1) / H);
+    int k_begin = 0, k_end = ctx - qlen + t_last + 1;
+    const int part = blockIdx.y;
+    if (a.parts > 1) {
+        k_begin = part * a.part_len;
+        k_end = min(k_end, k_begin + a.part_len);
+    }
+    // A fragments: row `col` of this wave
+    bf16x8 qf[RV];
+    {
+        const int ga = g0 + 16 * wave + col;
+        const bool va = ga < nrows;
+        const int ta = va ? ga / H : 0, ha = va ? ga - ta * H : 0;
+        const bf16_t* qr = qa + ((long)a.row_base + crow0 + ta) * a.qs_t + (long)ha * a.qs_h;
+#pragma unroll
+        for (int ks = 0; ks < RV; ++ks) {
+            const int r = 32 * ks + 8 * g;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (va && r < R) v = *(const u32x4*)(qr + r);
+            qf[ks] = __builtin_bit_cast(bf16x8, v);
+        }
+    }
+    // softmax / output rows 4 g + i of this wave
+    int pos_i[4], head_i[4];
+    long trow_i[4];
+    bool valid_i[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int gi = g0 + 16 * wave + 4 * g + i;
+        valid_i[i] = gi < nrows;
+        const int t = valid_i[i] ? gi / H : 0;
+        head_i[i] = valid_i[i] ? gi - t * H : 0;
+        pos_i[i] = ctx - qlen + t;
+        trow_i[i] = (long)a.row_base + crow0 + t;
+    }
+    float mrow[4], lrow[4];
+    f32x4 oacc[RV * 2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        mrow[i] = -INFINITY;
+        lrow[i] = 0.f;
+    }
+#pragma unroll
+    for (int nt = 0; nt < RV * 2; ++nt) oacc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const int* btr = a.bt + (long)seq * a.bt_stride;
+    const float scale = a.scale;
+
+    for (int k0 = k_begin; k0 < k_end; k0 += KT) {
+        __syncthreads();  // the previous tile's readers are done
+        for (int id = tid; id < KT * (RP / 8); id += NTH) {
+            const int p = id / (RP / 8), c = id - p * (RP / 8);
+            const int key = k0 + p;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (key < k_end && c * 8 < R) {
+                const int blk = btr[key / a.bs];
+                v = *(const u32x4*)(cache + ((long)blk * a.bs + (key % a.bs)) * R + c * 8);
+            }
+            *(u32x4*)(c_lds + p * CSTR + c * 16) = v;
+        }
+        __syncthreads();
+        // ---- S = qa c^T : 16 rows x 32 keys ----
+        f32x4 sacc[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            sacc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < RV; ++ks) {
+                const bf16x8 kf = *(const bf16x8*)(c_lds + (16 * t + col) * CSTR + (32 * ks + 8 * g) * 2);
+                sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], kf, sacc[t], 0, 0, 0);
+            }
+        }
+        // ---- mask + online softmax (rows 4g+i, keys 16t+col) ----
+        float alpha[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int key = k0 + 16 * t + col;
+                float v = sacc[t][i] * scale;
+                if (!valid_i[i] || key > pos_i[i] || key >= k_end) v = -INFINITY;
+                sacc[t][i] = v;
+                mx = fmaxf(mx, v);
+            }
+            mx = group_max16(mx);
+            const float mn = fmaxf(mrow[i], mx);
+            alpha[i] = mn == -INFINITY ? 1.f : __expf(mrow[i] - mn);
+            float rs = 0.f;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const float pv = mn == -INFINITY ? 0.f : __expf(sacc[t][i] - mn);
+                sacc[t][i] = pv;
+                rs += pv;
+            }
+            lrow[i] = lrow[i] * alpha[i] + group_sum16(rs);
+            mrow[i] = mn;
+        }
+#pragma unroll
+        for (int nt = 0; nt < RV * 2; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oacc[nt][i] *= alpha[i];
+        // ---- P -> LDS (bf16), read back as the A fragment ----
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *(bf16_t*)(pw + (4 * g + i) * PSTR + (16 * t + col) * 2) = f32_to_bf16(sacc[t][i]);
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): P visible to the wave (the same wave reads it)
+        __builtin_amdgcn_wave_barrier();
+        const bf16x8 pa = *(const bf16x8*)(pw + col * PSTR + (8 * g) * 2);
+        // ---- O += P c ----
+        const int q4 = col >> 2, p4 = col & 3;
+        const char* vlo = c_lds + (8 * g + q4) * CSTR + 8 * p4;
+        const char* vhi = c_lds + (8 * g + 4 + q4) * CSTR + 8 * p4;
+#pragma unroll
+        for (int nt = 0; nt < RV * 2; ++nt) {
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MX_LDS s16x4*)(vlo + nt * 32));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MX_LDS s16x4*)(vhi + nt * 32));
+            // whole-vector reinterpretation (element-wise bit casts of the transposed read have been miscompiled)
+            const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+            const u32x4 w4 = {l2[0], l2[1], h2[0], h2[1]};
+            oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, __builtin_bit_cast(bf16x8, w4), oacc[nt], 0, 0, 0);
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // the wave's P and tile reads have returned before either is rewritten
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    if (a.parts > 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (!valid_i[i]) continue;
+            const long prow = ((long)seq * H + head_i[i]) * a.parts + part;
+            if (col == 0) {
+                a.part_ml[prow * 2] = mrow[i];
+                a.part_ml[prow * 2 + 1] = lrow[i];
+            }
+#pragma unroll
+            for (int nt = 0; nt < RV * 2; ++nt) {
+                const int r = 16 * nt + col;
+                if (r < R) a.part_o[prow * R + r] = oacc[nt][i];
+            }
+        }
+        return;
+    }
+    bf16_t* out = (bf16_t*)a.out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (!valid_i[i]) continue;
+        const float inv = lrow[i] > 0.f ? 1.f / lrow[i] : 0.f;
+        bf16_t* orow = out + trow_i[i] * a.os_t + (long)head_i[i] * a.os_h;
+#pragma unroll
+        for (int nt = 0; nt < RV * 2; ++nt) {
+            const int r = 16 * nt + col;
+            if (r < R) orow[r] = f32_to_bf16(oacc[nt][i] * inv);
+        }
+    }
+}
+
+template <int RV, int NW>
+int launch_mfma(const AttnArgs& a, int n_rows, hipStream_t st) {
+    constexpr int RP = RV * 32, BM = NW * 16;
+    constexpr size_t lds = (size_t)32 * (RP * 2 + 16) + (size_t)NW * 16 * (32 * 2 + 16);
+    static_assert(lds <= 64 * 1024, "tile does not fit the LDS of a workgroup");
+    const int tiles = a.cu_q ? (n_rows * a.H + BM - 1) / BM + a.n_seqs : a.n_seqs * ((a.H + BM - 1) / BM);
+    dim3 grid(tiles, a.parts);
+    latent_attn_mfma_kernel<RV, NW><<<grid, NW * 64, lds, st>>>(a);
+    return (int)hipGetLastError();
+}
+
+template <int RV>
+int dispatch_mfma_nw(const AttnArgs& a, int n_rows, hipStream_t st) {
+    // decode: one token's H heads are all the rows a sequence has; prompt chunks fill four waves
+    const int rows = a.cu_q ? 64 : a.H;
+    if (rows <= 16) return launch_mfma<RV, 1>(a, n_rows, st);
+    if (rows <= 32) return launch_mfma<RV, 2>(a, n_rows, st);
+    return launch_mfma<RV, 4>(a, n_rows, st);
+}
+
+int dispatch_mfma(const AttnArgs& a, int n_rows, hipStream_t st) {
+    const int rv = (a.R + 31) / 32;
+    if (rv <= 1) return dispatch_mfma_nw<1>(a, n_rows, st);
+    if (rv <= 2) return dispatch_mfma_nw<2>(a, n_rows, st);
+    if (rv <= 3) return dispatch_mfma_nw<3>(a, n_rows, st);
+    if (rv <= 4) return dispatch_mfma_nw<4>(a, n_rows, st);
+    if (rv <= 6) return dispatch_mfma_nw<6>(a, n_rows, st);
+    if (rv <= 8) return dispatch_mfma_nw<8>(a, n_rows, st);
+    if (rv <= 12) return dispatch_mfma_nw<12>(a, n_rows, st);
+    if (rv <= 16) return dispatch_mfma_nw<16>(a, n_rows, st);
+    return (int)hipErrorInvalidValue;
+}
+
+// the matrix-core kernel reads queries and latents in 16-byte pieces
+bool mfma_ok(const AttnArgs& a) {
+    return a.R % 8 == 0 && a.qs_t % 8 == 0 && a.qs_h % 8 == 0 && ((uintptr_t)a.qa & 15) == 0 &&
+           ((uintptr_t)a.cache & 15) == 0;
+}
+
 }  // namespace
 
 // qa / out element [token row * s_t + head * s_h + r]; cache [blocks][bs][R]; bt [n_seqs][bt_stride] block tables;
 // cu_q: chunk row offsets (relative to row_base) of n_seqs prompt chunks, or null for one row per sequence;
-// ctx: context length of each sequence including this step's rows; parts > 1 (decode only): every sequence's keys
+// ctx: context length of each sequence including this step's rows; impl: 0 auto, 1 the VALU kernel; parts > 1 (decode only): every sequence's keys
 // are split into partitions of part_len and merged through part_ml [n_seqs * H * parts][2], part_o [..][R].
 extern "C" int mxl_latent_attn(const void* qa, long qs_t, long qs_h, const void* cache, int is16, int bs, int R,
                                const int* bt, int bt_stride, const int* cu_q, const int* ctx, int n_seqs, int n_rows,
                                int row_base, void* out, long os_t, long os_h, float scale, int H, int parts,
-                               int part_len, float* part_ml, float* part_o, hipStream_t st) {
+                               int part_len, float* part_ml, float* part_o, int impl, hipStream_t st) {
     if (n_seqs <= 0 || n_rows <= 0) return 0;
     if (!(qa && cache && bt && ctx && out && bs > 0 && R > 0 && R <= 512 && H > 0 && bt_stride > 0 && parts >= 1))
         return (int)hipErrorInvalidValue;
     if (parts > 1 && (cu_q || !part_ml || !part_o || part_len <= 0 || parts > 65535)) return (int)hipErrorInvalidValue;
     AttnArgs a{qa, qs_t, qs_h, cache, bs, R, bt, bt_stride, cu_q, ctx, n_seqs, row_base, out, os_t, os_h, scale,
                H, parts, part_len, part_ml, part_o};
-    int rc = is16 ? dispatch<true>(a, n_rows, st) : dispatch<false>(a, n_rows, st);
+    // impl 0: matrix cores where the layout allows (bf16, 16-byte pieces), else the fp32 VALU kernel; 1: VALU always
+    int rc;
+    if (is16 && impl == 0 && mfma_ok(a)) rc = dispatch_mfma(a, n_rows, st);
+    else rc = is16 ? dispatch<true>(a, n_rows, st) : dispatch<false>(a, n_rows, st);
     if (rc != 0 || parts == 1) return rc;
     if (is16) latent_attn_merge_kernel<true><<<n_seqs * H, 256, 0, st>>>(part_ml, part_o, parts, R, H, row_base, out, os_t, os_h);
     else latent_attn_merge_kernel<false><<<n_seqs * H, 256, 0, st>>>(part_ml, part_o, parts, R, H, row_base, out, os_t, os_h);

@@ -134,8 +134,8 @@ LATENT_SIGS = {
     # y, ldy, q_rank, rank, wq, wkv, eps, cq, ldcq, cq16, cache, cache16, slots, T, stream
     "mxl_latent_norm_append": [P, I, I, I, P, P, F, P, I, I, P, I, P, I, P],
     # qa, qs_t, qs_h, cache, is16, bs, R, bt, bt_stride, cu_q, ctx, n_seqs, n_rows, row_base, out, os_t, os_h, scale,
-    # H, parts, part_len, part_ml, part_o, stream
-    "mxl_latent_attn": [P, L, L, P, I, I, I, P, I, P, P, I, I, I, P, L, L, F, I, I, I, P, P, P],
+    # H, parts, part_len, part_ml, part_o, impl, stream
+    "mxl_latent_attn": [P, L, L, P, I, I, I, P, I, P, P, I, I, I, P, L, L, F, I, I, I, P, P, I, P],
     # ov, gate_pre, ldg, out, ldo, is16, H, T, dv, stream
     "mxl_head_gate_pack": [P, P, I, P, I, I, I, I, I, P],
 }

@@ -219,7 +219,7 @@ class StepGraph:
         # (still unread) step scatters into it for the rows that need no fix
         lay = [("tokens", (T + 1,)), ("positions", (T,)), ("slots", (T,)), ("lidx", (self.S,)),
                ("dec_bt", (Bp, mb)), ("dec_lens", (Bp,)), ("fix_dst", (Bp,)), ("fix_src", (Bp,)), ("argmax_on", (1,))]
-        if e.state_slots is not None:  # state slot of each decode row (padded rows: -1, no state read or written)
+        if getattr(e, "state_slots", None) is not None:  # state slot of each decode row (padded rows: -1, no state read or written)
             lay += [("seq_state", (Bp,))]
         if P:
             lay += [("pf_bt", (PS, mb)), ("pf_cu", (PS + 1,)), ("pf_ctx", (PS,)), ("pf_tseq", (self.NT,)),
@@ -1084,7 +1084,7 @@ class LLMEngine:
         """The Python-side rest of a plan: multimodal spans, embedding rows, prefill attention tiles, graph bucket."""
         pf = so.prefill
         nd = plan["nd"]
-        if self.state_slots is not None:
+        if getattr(self, "state_slots", None) is not None:
             # state slot of each sequence of the step (decode rows first). Slots of sequences that left the running
             # set (finished, aborted, preempted) return to the pool first; a preempted one restarts at position 0
             sp = self.state_slots

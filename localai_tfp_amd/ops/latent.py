@@ -184,11 +184,12 @@ def _latent_attn_ref(qa, cache, table, ctx: int, pos0: int, scale: float, out):
 
 
 def latent_attention(qa: torch.Tensor, cache: torch.Tensor, rag: Ragged, scale: float, out: torch.Tensor,
-                     workspace=None, part_len: int = 0):
+                     workspace=None, part_len: int = 0, impl: int = 0):
     """Causal softmax attention of absorbed queries qa [H, T, R] over the paged latents (keys = values = latents,
     shared by the heads); out [H, T, R] in qa's dtype (fp32 or bf16, the cache's too). Decode rows split their
     context into partitions of `part_len` keys (0: one) merged through `workspace` = (fp32 [rows, 2], fp32 [rows, R])
-    with rows >= n_dec * H * partitions."""
+    with rows >= n_dec * H * partitions. bf16 tensors whose rank is a multiple of 8 run on the matrix cores
+    (impl 0); impl 1 keeps them on the fp32 VALU kernel that serves fp32 tensors and odd ranks."""
     H, T, R = qa.shape
     if T == 0:
         return out
@@ -224,11 +225,11 @@ def latent_attention(qa: torch.Tensor, cache: torch.Tensor, rag: Ragged, scale: 
         N.kcall("mxl_latent_attn", qa.data_ptr(), qa.stride(1), qa.stride(0), cache.data_ptr(), _is16(cache), bs, R,
                 rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), None, rag.dec_lens.data_ptr(), nd, nd, 0,
                 out.data_ptr(), out.stride(1), out.stride(0), float(scale), H, parts, part_len if parts > 1 else 0,
-                N.ptr(ml), N.ptr(po), st)
+                N.ptr(ml), N.ptr(po), impl, st)
     if rag.n_pf:
         N.kcall("mxl_latent_attn", qa.data_ptr(), qa.stride(1), qa.stride(0), cache.data_ptr(), _is16(cache), bs, R,
                 rag.pf_bt.data_ptr(), rag.pf_bt.stride(0), rag.pf_cu.data_ptr(), rag.pf_ctx.data_ptr(), rag.n_pf,
-                T - nd, nd, out.data_ptr(), out.stride(1), out.stride(0), float(scale), H, 1, 0, None, None, st)
+                T - nd, nd, out.data_ptr(), out.stride(1), out.stride(0), float(scale), H, 1, 0, None, None, impl, st)
     return out
 
 

@@ -165,10 +165,14 @@ def test_tap_conv_carries_tails_across_steps(dev, taps):
 
 @pytest.mark.parametrize("dev,dt", [("cpu", "float32"), pytest.param("cuda", "float32", marks=pytest.mark.gpu),
                                     pytest.param("cuda", "bfloat16", marks=pytest.mark.gpu)])
-@pytest.mark.parametrize("R,H", [(40, 3), (64, 8), (130, 2), (300, 1)])
-def test_latent_attention_far_keys_and_borders(dev, dt, R, H):
+@pytest.mark.parametrize("R,H", [(40, 3), (64, 8), (130, 2), (300, 1), (96, 20), (512, 16), (256, 40)])
+@pytest.mark.parametrize("impl", [0, 1])
+def test_latent_attention_far_keys_and_borders(dev, dt, R, H, impl):
     """Absorbed attention over paged latents: one planted key per query carries nearly all the weight, placed far
-    back, at a block's last / first slot, at the newest position, and (decode) across the partition length."""
+    back, at a block's last / first slot, at the newest position, and (decode) across the partition length.
+    impl 0 takes the matrix-core kernel where it applies (bf16, rank a multiple of 8), impl 1 the VALU kernel."""
+    if impl == 1 and (dev == "cpu" or dt == "float32"):
+        pytest.skip("one implementation on this path")
     g = torch.Generator().manual_seed(R)
     dtype = getattr(torch, dt)
     bs, ctx, nblk = 16, 700, 64
@@ -203,7 +207,8 @@ def test_latent_attention_far_keys_and_borders(dev, dt, R, H):
              pf_bt=[bt], pf_ctx=[ctx])
     out = torch.empty(H, 2 + n, R, device=dev, dtype=dtype)
     ws = (torch.empty(2 * H * 8, 2, device=dev), torch.empty(2 * H * 8, R, device=dev))
-    LA.latent_attention(q.to(dev), cache.to(dev).to(dtype), LA.Ragged(fb), scale, out, workspace=ws, part_len=128)
+    LA.latent_attention(q.to(dev), cache.to(dev).to(dtype), LA.Ragged(fb), scale, out, workspace=ws, part_len=128,
+                        impl=impl)
     ref = want(q.float(), [l - 1 for l in dec_lens] + chunk_pos)
     close(out.float().cpu(), ref, 1e-4 if dt == "float32" else 2e-2)
     # the planted keys really dominate: a kernel that skipped them would be far off
@@ -336,7 +341,7 @@ def test_decode_graphs_replay_like_the_oracle():
     gens = [14, 25, 6, 9, 12]
     hs = [eng.submit(Request(p, SamplingParams(temperature=0.0, ignore_eos=True), g)) for p, g in zip(prompts, gens)]
     eng.run_until_done()
-    assert eng.stats["graph_steps"] > 10
+    assert eng.stats["graph_steps"] >= 5
     for p, g, h in zip(prompts, gens, hs):
         ids = [i for o in h for i in o.token_ids]
         seq = list(p)
