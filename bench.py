@@ -101,6 +101,8 @@ def parse():
                          "family beside the Llama graph at equal layer sizes (random bf16 / f16 weights, one GPU)")
     ap.add_argument("--arch-sizes", default="1b,7b", help="--arch-bench: comma list of layer sizes (1b, 7b)")
     ap.add_argument("--arch-layers", type=int, default=4, help="--arch-bench: layers per model")
+    ap.add_argument("--arch-models", default="", help="--arch-bench: comma list to restrict the models (vosotar, llama-f16)")
+    ap.add_argument("--arch-batches", default="1,32", help="--arch-bench: decode batch sizes")
     return ap.parse_args()
 
 
@@ -252,8 +254,10 @@ def run_arch_bench(args) -> int:
     rng = np.random.default_rng(0)
     for sz in [x for x in args.arch_sizes.split(",") if x]:
         for name, make in models(sz):
+            if args.arch_models and name not in args.arch_models.split(","):
+                continue
             model = make()
-            for B in (1, 32):
+            for B in [int(x) for x in args.arch_batches.split(",") if x]:
                 ec = EngineConfig(max_num_seqs=B, max_batched_tokens=P, max_model_len=P + G + 64, block_size=16,
                                   num_blocks=(B * (P + G + 64)) // 16 + 64, enable_prefix_cache=False,
                                   use_graphs=not args.no_graphs)

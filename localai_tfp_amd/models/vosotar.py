@@ -186,9 +186,12 @@ class VosotarWorkspace:
         self.act = torch.empty((T * ffm,), **md)
         self.hs = torch.empty((S, C), **md)
         self.logits = torch.empty((S, cfg.vocab), **f32)
+        # partial results of decode rows whose keys are split into partitions: room for every sequence at
+        # `max_parts` partitions, and for a lone sequence split finely enough to cover the chip
         hmax, rmax = max(m.heads for m in ms), max(m.kv_rank for m in ms)
-        self.part_ml = torch.empty((max_seqs * hmax * max_parts, 2), **f32)
-        self.part_o = torch.empty((max_seqs * hmax * max_parts, rmax), **f32)
+        rows = hmax * max(max_seqs * max_parts, 256)
+        self.part_ml = torch.empty((rows, 2), **f32)
+        self.part_o = torch.empty((rows, rmax), **f32)
 
 
 class VosotarModel:
@@ -196,7 +199,16 @@ class VosotarModel:
     tp_size = 1
     n_kv = 1
     n_heads = 1
-    DECODE_PART = 512  # keys per decode partition once a context is longer than this
+    DECODE_WGS = 512  # decode attention: workgroups to aim for when splitting contexts into key partitions
+
+    def decode_part_len(self, n_dec: int, heads: int, max_len: int) -> int:
+        """Keys per partition of the decode attention: a workgroup holds up to 64 (token, head) rows of one
+        sequence, so few sequences with long contexts are split finely (down to 64 keys) to cover the CUs, and
+        large batches coarsely (fewer partials to merge)."""
+        wgs = max(1, n_dec * -(-heads // 64))
+        want = max(1, self.DECODE_WGS // wgs)  # partitions per sequence
+        per = -(-max(1, max_len) // want)
+        return max(64, -(-per // 32) * 32)
 
     def __init__(self, cfg: VosotarConfig, device="cpu", dtype=None):
         self.cfg = cfg
@@ -332,7 +344,7 @@ class VosotarModel:
             torch.bmm(q.view(T, H, d).transpose(0, 1), W.uk, out=qa)
             ol = ws.ol[:H * T * R].view(H, T, R)
             LA.latent_attention(qa, lat, rag, mx.scale, ol, workspace=(ws.part_ml, ws.part_o),
-                                part_len=self.DECODE_PART)
+                                part_len=self.decode_part_len(rag.n_dec, H, rag.dec_max_len) if rag.n_dec else 0)
             ov = ws.ov[:H * T * dv].view(H, T, dv)
             _bmm_f32(ol, W.uvt, ov)
             att = ws.att[:T * H * dv].view(T, H * dv)

@@ -219,8 +219,10 @@ def latent_attention(qa: torch.Tensor, cache: torch.Tensor, rag: Ragged, scale: 
         parts = 1
         if part_len and workspace is not None and rag.dec_max_len > part_len:
             parts = -(-rag.dec_max_len // part_len)
-            if nd * H * parts > workspace[0].shape[0]:
-                parts = 1
+            room = workspace[0].shape[0] // (nd * H)  # partitions the partial-result buffers hold per row
+            if parts > room:
+                parts = max(1, room)
+                part_len = -(-(-(-rag.dec_max_len // parts)) // 32) * 32
         ml, po = (workspace[0], workspace[1]) if parts > 1 else (None, None)
         N.kcall("mxl_latent_attn", qa.data_ptr(), qa.stride(1), qa.stride(0), cache.data_ptr(), _is16(cache), bs, R,
                 rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), None, rag.dec_lens.data_ptr(), nd, nd, 0,
