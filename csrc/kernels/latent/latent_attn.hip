@@ -207,27 +207,45 @@ __global__ __launch_bounds__(BM * 8) void latent_attn_kernel(AttnArgs a) {
         }
 }
 
-// one block per (sequence, head): out = sum_p e^(m_p - M) o_p / sum_p e^(m_p - M) l_p
+// one block per (sequence, head): out = sum_p e^(m_p - M) o_p / sum_p e^(m_p - M) l_p. The partitions' weights are
+// worked out once into LDS (parts <= 1024), then every thread sums its columns over the partitions.
 template <bool B16>
 __global__ __launch_bounds__(256) void latent_attn_merge_kernel(const float* part_ml, const float* part_o, int parts,
                                                                 int R, int H, int row_base, void* out, long os_t,
                                                                 long os_h) {
+    __shared__ float wgt[1024];
+    __shared__ float red[8];
     const int seq = blockIdx.x / H, hh = blockIdx.x - seq * H;
     const long p0 = (long)blockIdx.x * parts;
-    float M = -INFINITY;
-    for (int p = 0; p < parts; ++p) M = fmaxf(M, part_ml[(p0 + p) * 2]);
-    float L = 0.f;
-    for (int p = 0; p < parts; ++p) {
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    float mloc = -INFINITY;
+    for (int p = tid; p < parts; p += 256) {
         const float mp = part_ml[(p0 + p) * 2];
-        if (mp != -INFINITY) L += __expf(mp - M) * part_ml[(p0 + p) * 2 + 1];
+        wgt[p] = mp;
+        mloc = fmaxf(mloc, mp);
     }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mloc = fmaxf(mloc, __shfl_xor(mloc, o, 64));
+    if (lane == 0) red[wv] = mloc;
+    __syncthreads();
+    const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float lloc = 0.f;
+    for (int p = tid; p < parts; p += 256) {
+        const float mp = wgt[p];
+        const float w = mp == -INFINITY ? 0.f : __expf(mp - M);
+        wgt[p] = w;
+        lloc += w * part_ml[(p0 + p) * 2 + 1];
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) lloc += __shfl_xor(lloc, o, 64);
+    if (lane == 0) red[4 + wv] = lloc;
+    __syncthreads();
+    const float L = red[4] + red[5] + red[6] + red[7];
     const float inv = L > 0.f ? 1.f / L : 0.f;
-    for (int c = threadIdx.x; c < R; c += 256) {
+    for (int c = tid; c < R; c += 256) {
         float o = 0.f;
-        for (int p = 0; p < parts; ++p) {
-            const float mp = part_ml[(p0 + p) * 2];
-            if (mp != -INFINITY) o += __expf(mp - M) * part_o[(p0 + p) * R + c];
-        }
+#pragma unroll 4
+        for (int p = 0; p < parts; ++p) o += wgt[p] * part_o[(p0 + p) * R + c];
         stf<B16>(out, ((long)row_base + seq) * os_t + (long)hh * os_h + c, o * inv);
     }
 }
@@ -365,15 +383,27 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
 
     for (int k0 = k_begin; k0 < k_end; k0 += KT) {
         __syncthreads();  // the previous tile's readers are done
-        for (int id = tid; id < KT * (RP / 8); id += NTH) {
-            const int p = id / (RP / 8), c = id - p * (RP / 8);
-            const int key = k0 + p;
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (key < k_end && c * 8 < R) {
-                const int blk = btr[key / a.bs];
-                v = *(const u32x4*)(cache + ((long)blk * a.bs + (key % a.bs)) * R + c * 8);
+        // the tile's 16-byte pieces, UB loads in flight per thread before the first one is stored
+        constexpr int CPK = RP / 8, TOTAL = KT * CPK, UB = 8;
+        for (int base = 0; base < TOTAL; base += NTH * UB) {
+            u32x4 v[UB];
+#pragma unroll
+            for (int u = 0; u < UB; ++u) {
+                const int id = base + u * NTH + tid;
+                const int p = id / CPK, c = id - p * CPK;
+                const int key = k0 + p;
+                v[u] = (u32x4){0u, 0u, 0u, 0u};
+                if (id < TOTAL && key < k_end && c * 8 < R) {
+                    const int blk = btr[key / a.bs];
+                    v[u] = *(const u32x4*)(cache + ((long)blk * a.bs + (key % a.bs)) * R + c * 8);
+                }
             }
-            *(u32x4*)(c_lds + p * CSTR + c * 16) = v;
+#pragma unroll
+            for (int u = 0; u < UB; ++u) {
+                const int id = base + u * NTH + tid;
+                const int p = id / CPK, c = id - p * CPK;
+                if (id < TOTAL) *(u32x4*)(c_lds + p * CSTR + c * 16) = v[u];
+            }
         }
         __syncthreads();
         // ---- S = qa c^T : 16 rows x 32 keys ----
@@ -526,7 +556,7 @@ extern "C" int mxl_latent_attn(const void* qa, long qs_t, long qs_h, const void*
     if (n_seqs <= 0 || n_rows <= 0) return 0;
     if (!(qa && cache && bt && ctx && out && bs > 0 && R > 0 && R <= 512 && H > 0 && bt_stride > 0 && parts >= 1))
         return (int)hipErrorInvalidValue;
-    if (parts > 1 && (cu_q || !part_ml || !part_o || part_len <= 0 || parts > 65535)) return (int)hipErrorInvalidValue;
+    if (parts > 1 && (cu_q || !part_ml || !part_o || part_len <= 0 || parts > 1024)) return (int)hipErrorInvalidValue;
     AttnArgs a{qa, qs_t, qs_h, cache, bs, R, bt, bt_stride, cu_q, ctx, n_seqs, row_base, out, os_t, os_h, scale,
                H, parts, part_len, part_ml, part_o};
     // impl 0: matrix cores where the layout allows (bf16, 16-byte pieces), else the fp32 VALU kernel; 1: VALU always

@@ -61,19 +61,45 @@ __global__ __launch_bounds__(NT) void embed_norm_kernel(const void* table, int V
     for (int c = threadIdx.x; c < C; c += NT) out[(long)t * ldo + c] = ld_elem<B16>(table, base + c) * sc;
 }
 
+// rows of up to NT * RC numbers are read once and kept in registers between the statistics and the output pass
+constexpr int RC = 16;
+
 __global__ __launch_bounds__(NT) void scalar_norm_kernel(const float* x, int ldx, const int* rows, const float* g,
                                                          float eps, float* o32, int ld32, bf16_t* o16, int ld16,
                                                          int C) {
     __shared__ float red[NT / 64];
     const int i = blockIdx.x;
     const float* xr = x + (long)(rows ? rows[i] : i) * ldx;
+    const bool cached = C <= NT * RC;
+    float keep[RC];
     float ss = 0.f;
-    for (int c = threadIdx.x; c < C; c += NT) {
-        const float v = xr[c];
-        ss += v * v;
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {
+            const int c = threadIdx.x + k * NT;
+            keep[k] = c < C ? xr[c] : 0.f;
+            ss += keep[k] * keep[k];
+        }
+    } else {
+        for (int c = threadIdx.x; c < C; c += NT) {
+            const float v = xr[c];
+            ss += v * v;
+        }
     }
     ss = block_sum(ss, red);
     const float sc = g[0] / sqrtf(ss / (float)C + eps);
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {
+            const int c = threadIdx.x + k * NT;
+            if (c < C) {
+                const float v = keep[k] * sc;
+                if (o32) o32[(long)i * ld32 + c] = v;
+                if (o16) o16[(long)i * ld16 + c] = f32_to_bf16(v);
+            }
+        }
+        return;
+    }
     for (int c = threadIdx.x; c < C; c += NT) {
         const float v = xr[c] * sc;
         if (o32) o32[(long)i * ld32 + c] = v;
@@ -81,21 +107,42 @@ __global__ __launch_bounds__(NT) void scalar_norm_kernel(const float* x, int ldx
     }
 }
 
+// x += g * unit_rms(z), z = y * sigmoid(gate_pre + gate_bias)
 __global__ __launch_bounds__(NT) void gated_norm_add_kernel(float* x, int ldx, const float* y, int ldy,
-                                                            const float* gp, int ldg, const float* g, float eps,
-                                                            int C) {
+                                                            const float* gp, int ldg, const float* gb, const float* g,
+                                                            float eps, int C) {
     __shared__ float red[NT / 64];
     const int i = blockIdx.x;
     const float* yr = y + (long)i * ldy;
     const float* gr = gp + (long)i * ldg;
+    const bool cached = C <= NT * RC;
+    float keep[RC];
     float ss = 0.f;
-    for (int c = threadIdx.x; c < C; c += NT) {
-        const float z = yr[c] * sigmoidf_(gr[c]);
-        ss += z * z;
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {
+            const int c = threadIdx.x + k * NT;
+            keep[k] = c < C ? yr[c] * sigmoidf_(gr[c] + (gb ? gb[c] : 0.f)) : 0.f;
+            ss += keep[k] * keep[k];
+        }
+    } else {
+        for (int c = threadIdx.x; c < C; c += NT) {
+            const float z = yr[c] * sigmoidf_(gr[c] + (gb ? gb[c] : 0.f));
+            ss += z * z;
+        }
     }
     ss = block_sum(ss, red);
     const float sc = g[0] / sqrtf(ss / (float)C + eps);
-    for (int c = threadIdx.x; c < C; c += NT) x[(long)i * ldx + c] += yr[c] * sigmoidf_(gr[c]) * sc;
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {
+            const int c = threadIdx.x + k * NT;
+            if (c < C) x[(long)i * ldx + c] += keep[k] * sc;
+        }
+        return;
+    }
+    for (int c = threadIdx.x; c < C; c += NT)
+        x[(long)i * ldx + c] += yr[c] * sigmoidf_(gr[c] + (gb ? gb[c] : 0.f)) * sc;
 }
 
 template <bool B16>
@@ -228,11 +275,11 @@ extern "C" int mxl_scalar_norm(const float* x, int ldx, const int* rows, const f
     return (int)hipGetLastError();
 }
 
-extern "C" int mxl_gated_norm_add(float* x, int ldx, const float* y, int ldy, const float* gp, int ldg, const float* g,
-                                  float eps, int M, int C, hipStream_t st) {
+extern "C" int mxl_gated_norm_add(float* x, int ldx, const float* y, int ldy, const float* gp, int ldg, const float* gb,
+                                  const float* g, float eps, int M, int C, hipStream_t st) {
     if (M <= 0) return 0;
     MXL_CHECK(x && y && gp && g && C > 0 && ldx >= C && ldy >= C && ldg >= C);
-    gated_norm_add_kernel<<<M, NT, 0, st>>>(x, ldx, y, ldy, gp, ldg, g, eps, C);
+    gated_norm_add_kernel<<<M, NT, 0, st>>>(x, ldx, y, ldy, gp, ldg, gb, g, eps, C);
     return (int)hipGetLastError();
 }
 

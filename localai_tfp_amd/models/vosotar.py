@@ -4,16 +4,16 @@ causal convolution over each mixer's input.
 One layer on the fp32 residual x (T rows of a ragged engine step; g* are one-number gains):
 
     h    = g1 * unit_rms(x)                              (latent.hip scalar norm -> fp32 + GEMM operand)
-    gate = h W_rg1^T + b                                  (hipBLASLt, fp32 out)
+    gate = h W_rg1^T                                      (hipBLASLt, fp32 out; its bias joins in the gated add)
     hm   = h + tapconv(h)                                 (latent.hip; last taps-1 rows of h carried per sequence)
     y    = hm [W_dq | W_dkv | W_g]^T                      (one GEMM for the three projections that read hm)
     cq   = w_q * unit_rms(y[:, :q_rank]);  c = w_kv * unit_rms(y[:, q_rank:+rank]) -> paged latent pool
     qa   = (cq W_uq^T) per head times U_k                 (GEMM, then batched GEMM: absorbed queries [H, T, rank])
     o    = softmax(scale * qa . c_j) over j <= position, times c_j       (latent_attn.hip, keys = values = latents)
     att  = (o U_v^T) * sigmoid(y[:, gate columns]) per head              (batched GEMM, latent.hip pack)
-    x   += g1b * unit_rms((att W_o^T) * sigmoid(gate))    (GEMM, latent.hip gated norm add)
-    h2   = g2 * unit_rms(x);  u = h2 [W_up | W_rg2]^T + [0 | b2]
-    x   += g2b * unit_rms((relu(u_up)^2 W_down^T) * sigmoid(u_rg2))
+    x   += g1b * unit_rms((att W_o^T) * sigmoid(gate + b)) (GEMM, latent.hip gated norm add)
+    h2   = g2 * unit_rms(x);  u = h2 [W_up | W_rg2]^T
+    x   += g2b * unit_rms((relu(u_up)^2 W_down^T) * sigmoid(u_rg2 + b2))
 
 A layer entry may name another layer whose tensors it uses (`weights_of`); it still has its own latent pool and
 convolution tails. A layer without a feed-forward stops after the mixer. Sizes come from config.json, per layer.
@@ -142,7 +142,9 @@ class VosotarWeights:
     n2: torch.Tensor | None
     n2b: torch.Tensor | None
     canon: torch.Tensor  # [C, taps] fp32
-    rg1: Dense  # [C, C] + bias
+    rg1: Dense  # [C, C]; its bias joins in the gated add
+    rg1_b: torch.Tensor
+    rg2_b: torch.Tensor | None
     w_in: Dense  # rows: dq | dkv | g
     dq_norm: torch.Tensor
     dkv_norm: torch.Tensor
@@ -150,7 +152,7 @@ class VosotarWeights:
     uk: torch.Tensor  # [H, dim, rank]
     uvt: torch.Tensor  # [H, rank, vdim]
     o: Dense
-    up_rg2: Dense | None  # rows: up | rg2 (+ bias 0 | b2)
+    up_rg2: Dense | None  # rows: up | rg2
     down: Dense | None
 
 
@@ -279,16 +281,17 @@ class VosotarModel:
                               t(p + "mix.g", (H, C)).float()], 0)
             uk = t(p + "mix.uk", (H * d, R)).float().reshape(H, d, R)
             uv = t(p + "mix.uv", (H * dv, R)).float().reshape(H, dv, R)
-            up_rg2 = down = n2 = n2b = None
+            up_rg2 = down = n2 = n2b = rg2_b = None
             if L.ff is not None:
                 up_rg2 = Dense(torch.cat([t(p + "mlp.up", (L.ff, C)).float(), t(p + "rg2", (C, C)).float()], 0),
-                               torch.cat([torch.zeros(L.ff), t(p + "rg2.b", (C,)).float()]), dev, md)
+                               None, dev, md)
+                rg2_b = f32(p + "rg2.b", (C,))
                 down = Dense(t(p + "mlp.down", (C, L.ff)).float(), None, dev, md)
                 n2, n2b = one(p + "norm2"), one(p + "norm2b")
             m.weights[i] = VosotarWeights(
                 n1=one(p + "norm1"), n1b=one(p + "norm1b"), n2=n2, n2b=n2b,
                 canon=f32(p + "canon1", (C, cfg.taps)),
-                rg1=Dense(t(p + "rg1", (C, C)).float(), t(p + "rg1.b", (C,)).float(), dev, md),
+                rg1=Dense(t(p + "rg1", (C, C)).float(), None, dev, md), rg1_b=f32(p + "rg1.b", (C,)), rg2_b=rg2_b,
                 w_in=Dense(w_in, None, dev, md),
                 dq_norm=f32(p + "mix.dq.norm", (Rq,)), dkv_norm=f32(p + "mix.dkv.norm", (R,)),
                 uq=Dense(t(p + "mix.uq", (H * d, Rq)).float(), None, dev, md),
@@ -350,7 +353,7 @@ class VosotarModel:
             att = ws.att[:T * H * dv].view(T, H * dv)
             LA.head_gate_pack(ov, y_in[:, Rq + R:], att)
             W.o.into(att, y)
-            LA.gated_norm_add(x, y, gate, W.n1b, eps)
+            LA.gated_norm_add(x, y, gate, W.n1b, eps, W.rg1_b)
             # ---- feed-forward ----
             if L.ff is None:
                 continue
@@ -361,7 +364,7 @@ class VosotarModel:
             act = ws.act[:T * F_].view(T, F_)
             LA.relu2(u[:, :F_], act)
             W.down.into(act, y)
-            LA.gated_norm_add(x, y, u[:, F_:], W.n2b, eps)
+            LA.gated_norm_add(x, y, u[:, F_:], W.n2b, eps, W.rg2_b)
         if fb.stop_layer is not None:
             return x
         # ---- head ----

@@ -90,17 +90,20 @@ def scalar_rmsnorm(x: torch.Tensor, g: torch.Tensor, eps: float, out32: torch.Te
             M, C, N.stream_ptr())
 
 
-def gated_norm_add(x: torch.Tensor, y: torch.Tensor, gate_pre: torch.Tensor, g: torch.Tensor, eps: float):
-    """x += unit_rms(y * sigmoid(gate_pre)) * g on fp32 rows [M, C]; gate_pre may be a column slice."""
+def gated_norm_add(x: torch.Tensor, y: torch.Tensor, gate_pre: torch.Tensor, g: torch.Tensor, eps: float,
+                   gate_bias: torch.Tensor | None = None):
+    """x += unit_rms(y * sigmoid(gate_pre + gate_bias)) * g on fp32 rows [M, C]; gate_pre may be a column slice,
+    gate_bias is fp32 [C]."""
     M, C = y.shape
     if M == 0:
         return x
     if not x.is_cuda:
-        z = y.float() * torch.sigmoid(gate_pre.float())
+        gp = gate_pre.float() + gate_bias if gate_bias is not None else gate_pre.float()
+        z = y.float() * torch.sigmoid(gp)
         x.add_(z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps) * g.float())
         return x
     N.kcall("mxl_gated_norm_add", x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0), gate_pre.data_ptr(),
-            gate_pre.stride(0), g.data_ptr(), float(eps), M, C, N.stream_ptr())
+            gate_pre.stride(0), N.ptr(gate_bias), g.data_ptr(), float(eps), M, C, N.stream_ptr())
     return x
 
 

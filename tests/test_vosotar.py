@@ -112,8 +112,17 @@ def test_norms_gate_and_activation(dev):
     # x += gain * unit_rms(y * sigmoid(gate)); the gate is a column slice of a wider buffer
     y, wide = torch.randn(M, C, generator=g), torch.randn(M, C + 9, generator=g)
     res = x.clone().to(dev)
-    LA.gated_norm_add(res, y.to(dev), wide.to(dev)[:, 9:], gain.to(dev), eps)
-    close(res.cpu(), x.double() + O.scalar_norm(y.double() * torch.sigmoid(wide.double()[:, 9:]), gain, eps), 1e-5)
+    bias = torch.randn(C, generator=g)
+    LA.gated_norm_add(res, y.to(dev), wide.to(dev)[:, 9:], gain.to(dev), eps, bias.to(dev))
+    close(res.cpu(), x.double() + O.scalar_norm(y.double() * torch.sigmoid(wide.double()[:, 9:] + bias.double()),
+                                                gain, eps), 1e-5)
+    for C2 in (4100, 5000):  # rows wider than the kernels keep in registers
+        x2, y2, g2 = (torch.randn(3, C2, generator=g) for _ in range(3))
+        r2, n2 = x2.clone().to(dev), torch.empty(3, C2, device=dev)
+        LA.gated_norm_add(r2, y2.to(dev), g2.to(dev), gain.to(dev), eps)
+        close(r2.cpu(), x2.double() + O.scalar_norm(y2.double() * torch.sigmoid(g2.double()), gain, eps), 1e-5)
+        LA.scalar_rmsnorm(x2.to(dev), gain.to(dev), eps, out32=n2)
+        close(n2.cpu(), O.scalar_norm(x2.double(), gain, eps), 1e-5)
     # squared relu on a column slice
     a = torch.empty(M, C, device=dev)
     LA.relu2(wide.to(dev)[:, :C], a)
