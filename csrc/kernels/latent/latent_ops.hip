@@ -116,12 +116,14 @@ __global__ __launch_bounds__(NT) void gated_norm_add_kernel(float* x, int ldx, c
     const float* yr = y + (long)i * ldy;
     const float* gr = gp + (long)i * ldg;
     const bool cached = C <= NT * RC;
-    float keep[RC];
+    float keep[RC], xin[RC];
     float ss = 0.f;
     if (cached) {
+        // every load of the row (the residual too) is issued before the statistics: one memory round trip
 #pragma unroll
         for (int k = 0; k < RC; ++k) {
             const int c = threadIdx.x + k * NT;
+            xin[k] = c < C ? x[(long)i * ldx + c] : 0.f;
             keep[k] = c < C ? yr[c] * sigmoidf_(gr[c] + (gb ? gb[c] : 0.f)) : 0.f;
             ss += keep[k] * keep[k];
         }
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(NT) void gated_norm_add_kernel(float* x, int ldx, c
 #pragma unroll
         for (int k = 0; k < RC; ++k) {
             const int c = threadIdx.x + k * NT;
-            if (c < C) x[(long)i * ldx + c] += keep[k] * sc;
+            if (c < C) x[(long)i * ldx + c] = xin[k] + keep[k] * sc;
         }
         return;
     }

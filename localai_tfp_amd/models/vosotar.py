@@ -205,12 +205,12 @@ class VosotarModel:
 
     def decode_part_len(self, n_dec: int, heads: int, max_len: int) -> int:
         """Keys per partition of the decode attention: a workgroup holds up to 64 (token, head) rows of one
-        sequence, so few sequences with long contexts are split finely (down to 64 keys) to cover the CUs, and
+        sequence, so few sequences with long contexts are split finely (down to one 32-key tile) to cover the CUs, and
         large batches coarsely (fewer partials to merge)."""
         wgs = max(1, n_dec * -(-heads // 64))
         want = max(1, self.DECODE_WGS // wgs)  # partitions per sequence
         per = -(-max(1, max_len) // want)
-        return max(64, -(-per // 32) * 32)
+        return max(32, -(-per // 32) * 32)
 
     def __init__(self, cfg: VosotarConfig, device="cpu", dtype=None):
         self.cfg = cfg
