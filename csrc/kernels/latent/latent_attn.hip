@@ -381,31 +381,43 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
     const int* btr = a.bt + (long)seq * a.bt_stride;
     const float scale = a.scale;
 
-    for (int k0 = k_begin; k0 < k_end; k0 += KT) {
-        __syncthreads();  // the previous tile's readers are done
-        // the tile's 16-byte pieces, UB loads in flight per thread before the first one is stored
-        constexpr int CPK = RP / 8, TOTAL = KT * CPK, UB = 8;
-        for (int base = 0; base < TOTAL; base += NTH * UB) {
-            u32x4 v[UB];
+    // A tile is KT * CPK 16-byte pieces. Each thread's first UB pieces of the NEXT tile are requested before the
+    // current tile's products and stay in registers meanwhile (all of a tile when NTH * UB covers it); the rest
+    // is loaded UB pieces at a time once the tile's turn has come.
+    constexpr int CPK = RP / 8, TOTAL = KT * CPK, UB = (NW == 1 && RV > 8) ? 4 : 8;  // registers are full at RV 16
+    u32x4 pre[UB];
+    auto fetch = [&](int k0, int base, u32x4* v) {
 #pragma unroll
-            for (int u = 0; u < UB; ++u) {
-                const int id = base + u * NTH + tid;
-                const int p = id / CPK, c = id - p * CPK;
-                const int key = k0 + p;
-                v[u] = (u32x4){0u, 0u, 0u, 0u};
-                if (id < TOTAL && key < k_end && c * 8 < R) {
-                    const int blk = btr[key / a.bs];
-                    v[u] = *(const u32x4*)(cache + ((long)blk * a.bs + (key % a.bs)) * R + c * 8);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < UB; ++u) {
-                const int id = base + u * NTH + tid;
-                const int p = id / CPK, c = id - p * CPK;
-                if (id < TOTAL) *(u32x4*)(c_lds + p * CSTR + c * 16) = v[u];
+        for (int u = 0; u < UB; ++u) {
+            const int id = base + u * NTH + tid;
+            const int p = id / CPK, c = id - p * CPK;
+            const int key = k0 + p;
+            v[u] = (u32x4){0u, 0u, 0u, 0u};
+            if (id < TOTAL && key < k_end && c * 8 < R) {
+                const int blk = btr[key / a.bs];
+                v[u] = *(const u32x4*)(cache + ((long)blk * a.bs + (key % a.bs)) * R + c * 8);
             }
         }
+    };
+    auto stash = [&](int base, const u32x4* v) {
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+            const int id = base + u * NTH + tid;
+            const int p = id / CPK, c = id - p * CPK;
+            if (id < TOTAL) *(u32x4*)(c_lds + p * CSTR + c * 16) = v[u];
+        }
+    };
+    if (k_begin < k_end) fetch(k_begin, 0, pre);
+    for (int k0 = k_begin; k0 < k_end; k0 += KT) {
+        __syncthreads();  // the previous tile's readers are done
+        stash(0, pre);
+        for (int base = NTH * UB; base < TOTAL; base += NTH * UB) {
+            u32x4 v[UB];
+            fetch(k0, base, v);
+            stash(base, v);
+        }
         __syncthreads();
+        if (k0 + KT < k_end) fetch(k0 + KT, 0, pre);
         // ---- S = qa c^T : 16 rows x 32 keys ----
         f32x4 sacc[2];
 #pragma unroll
