@@ -322,7 +322,7 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
                 const int nt = (q * H + BM - 1) / BM;
                 if (tile < nt) {
                     seq = s;
-                    g0 = tile * BM;
+                    g0 = (nt - 1 - tile) * BM;  // a chunk's last rows see the most keys: their workgroups start first
                     qlen = q;
                     crow0 = a.cu_q[s];
                     break;
@@ -380,10 +380,12 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
     for (int nt = 0; nt < RV * 2; ++nt) oacc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
     const int* btr = a.bt + (long)seq * a.bt_stride;
     const float scale = a.scale;
+    const bool wave_active = g0 + 16 * wave < nrows;
 
     // A tile is KT * CPK 16-byte pieces. Each thread's first UB pieces of the NEXT tile are requested before the
     // current tile's products and stay in registers meanwhile (all of a tile when NTH * UB covers it); the rest
     // is loaded UB pieces at a time once the tile's turn has come.
+    const int bs_shift = (a.bs & (a.bs - 1)) == 0 ? __builtin_ctz(a.bs) : -1;
     constexpr int CPK = RP / 8, TOTAL = KT * CPK, UB = (NW == 1 && RV > 8) ? 4 : 8;  // registers are full at RV 16
     u32x4 pre[UB];
     auto fetch = [&](int k0, int base, u32x4* v) {
@@ -394,8 +396,10 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
             const int key = k0 + p;
             v[u] = (u32x4){0u, 0u, 0u, 0u};
             if (id < TOTAL && key < k_end && c * 8 < R) {
-                const int blk = btr[key / a.bs];
-                v[u] = *(const u32x4*)(cache + ((long)blk * a.bs + (key % a.bs)) * R + c * 8);
+                // block sizes are powers of two in practice: a shift instead of a division per piece
+                const int bi = bs_shift >= 0 ? key >> bs_shift : key / a.bs;
+                const int bo = key - bi * a.bs;
+                v[u] = *(const u32x4*)(cache + ((long)btr[bi] * a.bs + bo) * R + c * 8);
             }
         }
     };
@@ -418,6 +422,7 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
         }
         __syncthreads();
         if (k0 + KT < k_end) fetch(k0 + KT, 0, pre);
+        if (!wave_active) continue;  // a wave without rows only helps to fetch (the barriers are at the loop's top)
         // ---- S = qa c^T : 16 rows x 32 keys ----
         f32x4 sacc[2];
 #pragma unroll
@@ -455,10 +460,14 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
             lrow[i] = lrow[i] * alpha[i] + group_sum16(rs);
             mrow[i] = mn;
         }
+        // the running maxima settle after the first tiles: rescale only when some row's maximum moved
+        const bool moved = alpha[0] != 1.f || alpha[1] != 1.f || alpha[2] != 1.f || alpha[3] != 1.f;
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
 #pragma unroll
-        for (int nt = 0; nt < RV * 2; ++nt)
+            for (int nt = 0; nt < RV * 2; ++nt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) oacc[nt][i] *= alpha[i];
+                for (int i = 0; i < 4; ++i) oacc[nt][i] *= alpha[i];
+        }
         // ---- P -> LDS (bf16), read back as the A fragment ----
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -529,10 +538,10 @@ int launch_mfma(const AttnArgs& a, int n_rows, hipStream_t st) {
 
 template <int RV>
 int dispatch_mfma_nw(const AttnArgs& a, int n_rows, hipStream_t st) {
-    // decode: one token's H heads are all the rows a sequence has; prompt chunks fill four waves
-    const int rows = a.cu_q ? 64 : a.H;
-    if (rows <= 16) return launch_mfma<RV, 1>(a, n_rows, st);
-    if (rows <= 32) return launch_mfma<RV, 2>(a, n_rows, st);
+    // prompt chunks fill four waves. A decode row set is one token's H heads: up to 32 of them take two waves
+    // (the second only helps to fetch the key tiles when H <= 16), which leaves room for a second workgroup on the
+    // CU at the register budget of the widest ranks; more heads take four
+    if (!a.cu_q && a.H <= 32) return launch_mfma<RV, 2>(a, n_rows, st);
     return launch_mfma<RV, 4>(a, n_rows, st);
 }
 

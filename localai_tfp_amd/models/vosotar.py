@@ -207,7 +207,7 @@ class VosotarModel:
         """Keys per partition of the decode attention: a workgroup holds up to 64 (token, head) rows of one
         sequence, so few sequences with long contexts are split finely (down to one 32-key tile) to cover the CUs, and
         large batches coarsely (fewer partials to merge)."""
-        wgs = max(1, n_dec * -(-heads // 64))
+        wgs = max(1, n_dec * -(-heads // (32 if heads <= 32 else 64)))
         want = max(1, self.DECODE_WGS // wgs)  # partitions per sequence
         per = -(-max(1, max_len) // want)
         return max(32, -(-per // 32) * 32)
