@@ -90,10 +90,14 @@ class VosotarConfig:
             mlp = e.get("mlp")
             if mlp is not None and mlp.get("kind") != "dense":
                 raise ValueError(f"layer {i}: unknown feed-forward {mlp.get('kind')!r}")
-            wo = e.get("weights_of")
-            if wo is not None and not (0 <= int(wo) < len(d["layers"])) or wo is not None and \
-                    d["layers"][int(wo)].get("weights_of") is not None:
-                raise ValueError(f"layer {i}: weights_of must name a layer with tensors of its own")
+            wo, hops = e.get("weights_of"), 0
+            while wo is not None:  # follow a chain of borrowed layers to the one that has the tensors
+                if not 0 <= int(wo) < len(d["layers"]) or hops > len(d["layers"]):
+                    raise ValueError(f"layer {i}: weights_of does not lead to a layer with tensors of its own")
+                nxt = d["layers"][int(wo)].get("weights_of")
+                if nxt is None:
+                    break
+                wo, hops = nxt, hops + 1
             layers.append(VosotarLayerCfg(
                 LatentMixer(int(m["heads"]), int(m["dim"]), int(m["vdim"]), int(m["kv_rank"]), int(m["q_rank"]),
                             float(m["scale"])),
