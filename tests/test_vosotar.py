@@ -439,3 +439,20 @@ def test_served_through_the_llm_worker(tmp_path):
         if svc.engine is not None:
             svc.engine.shutdown()
         server.stop()
+
+
+@pytest.mark.parametrize("dev,dt,tol", RUNS)
+def test_layers_of_different_sizes(dev, dt, tol):
+    """Every layer with its own head count, head sizes, ranks and feed-forward width (one without any), a borrowed
+    layer in the middle: pools, workspaces and kernels take each layer's sizes, not the first one's."""
+    mk = lambda h, d, dv, r, rq, s, ff, wo=None: VO.VosotarLayerCfg(VO.LatentMixer(h, d, dv, r, rq, s), ff, wo)  # noqa: E731
+    cfg = VO.VosotarConfig(hidden=56, vocab=83, taps=4, rms_eps=1e-5, layers=[
+        mk(2, 16, 8, 24, 40, 0.3, 70), mk(5, 8, 20, 72, 12, 0.7, None), mk(2, 16, 8, 24, 40, 0.3, 70, 0),
+        mk(1, 40, 40, 8, 64, 0.2, 24)])
+    get = VO.synthetic_source(cfg, 17)
+    model = VO.VosotarModel.load(cfg, get, torch.device(dev), getattr(torch, dt))
+    t = toks(50, cfg.vocab, 4)
+    want = oracle(cfg, {k: get(k) for k in get.names}, t)
+    eng = engine(model, 64)
+    close(run_cuts(eng, "a", t, [50]), want, tol)
+    close(run_cuts(eng, "b", t, [17, 2, 1, 1, 20, 9]), want, tol)
