@@ -113,7 +113,7 @@ __global__ __launch_bounds__(BM * 8) void latent_attn_kernel(AttnArgs a) {
     const int* btr = a.bt + (long)seq * a.bt_stride;
 
     for (int k0 = k_begin; k0 < k_end; k0 += BN) {
-        __syncthreads();  // the previous tile's readers are done (and QA is written, first time round)
+        __syncthreads();  // the previous tile's readers are done (and QA is written, on the first pass)
         for (int i = tid; i < BN * RW; i += NTH) {
             const int j = i / RW, r = i - j * RW;
             const int key = k0 + j;

@@ -456,3 +456,26 @@ def test_layers_of_different_sizes(dev, dt, tol):
     eng = engine(model, 64)
     close(run_cuts(eng, "a", t, [50]), want, tol)
     close(run_cuts(eng, "b", t, [17, 2, 1, 1, 20, 9]), want, tol)
+
+
+@pytest.mark.parametrize("native", [False, True])
+def test_preempted_request_recomputes_its_state(native):
+    """A pool too small for both requests' growth: one is preempted, loses its blocks and state slot, and is
+    recomputed from position 0 later; both still produce the oracle's greedy tokens."""
+    cfg, tensors, model = build("cpu", "float32", seed=8, **SHAPES["odd"])
+    ec = EngineConfig(max_num_seqs=2, max_batched_tokens=64, max_model_len=128, block_size=16, num_blocks=8,
+                      use_graphs=False, native_scheduler=native, gemm_autotune=False)
+    eng = LLMEngine(model, ByteTokenizer(cfg.vocab), ec)
+    if native and not eng.native_sched:
+        pytest.skip("native runtime not built")
+    from localai_tfp_amd.engine.sequence import Request
+    prompts = [toks(30, cfg.vocab, 51), toks(28, cfg.vocab, 52)]
+    hs = [eng.submit(Request(p, SamplingParams(temperature=0.0, ignore_eos=True), 40)) for p in prompts]
+    eng.run_until_done()
+    assert eng.stats["preemptions"] > 0
+    for p, h in zip(prompts, hs):
+        ids = [i for o in h for i in o.token_ids]
+        seq = list(p)
+        for _ in range(40):
+            seq.append(int(oracle(cfg, tensors, seq)[-1].argmax()))
+        assert ids == seq[len(p):]
