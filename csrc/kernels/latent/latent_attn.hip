@@ -298,13 +298,7 @@ MX_DEV float group_sum16(float v) {
 
 template <int RV, int NW>
 __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
-    // LDS image of a tile: key rows of CSTR bytes. With rows 8 banks apart (32 bytes of padding) and, for rows
-    // 8..15 of every 16, the 16-byte piece index XOR-ed by 9 (the other half of the banks, and the other half of the
-    // row's 8-bank group), both the 16-byte score reads (16 keys per pass) and the transposed reads (4 keys x 32 bytes
-    // per 16-lane group, two groups per pass) are free of bank conflicts. The XOR needs the row's piece count to be a multiple of 16 (R_pad a multiple of 128).
-    constexpr int RP = RV * 32, KT = 32, PSTR = KT * 2 + 16, BM = NW * 16, NTH = NW * 64;
-    constexpr bool SWZ = RV % 4 == 0;
-    constexpr int CSTR = RP * 2 + (SWZ ? 32 : 16);
+    constexpr int RP = RV * 32, KT = 32, CSTR = RP * 2 + 16, PSTR = KT * 2 + 16, BM = NW * 16, NTH = NW * 64;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char* c_lds = smem;                                   // [KT][CSTR] bf16 latents of the tile
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, g = lane >> 4;
@@ -414,7 +408,7 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
         for (int u = 0; u < UB; ++u) {
             const int id = base + u * NTH + tid;
             const int p = id / CPK, c = id - p * CPK;
-            if (id < TOTAL) *(u32x4*)(c_lds + p * CSTR + (SWZ ? c ^ ((p & 8) | ((p & 8) >> 3)) : c) * 16) = v[u];
+            if (id < TOTAL) *(u32x4*)(c_lds + p * CSTR + c * 16) = v[u];
         }
     };
     if (k_begin < k_end) fetch(k_begin, 0, pre);
@@ -436,7 +430,7 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
             sacc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < RV; ++ks) {
-                const bf16x8 kf = *(const bf16x8*)(c_lds + (16 * t + col) * CSTR + (SWZ ? (4 * ks + g) ^ ((col & 8) | ((col & 8) >> 3)) : 4 * ks + g) * 16);
+                const bf16x8 kf = *(const bf16x8*)(c_lds + (16 * t + col) * CSTR + (32 * ks + 8 * g) * 2);
                 sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], kf, sacc[t], 0, 0, 0);
             }
         }
@@ -484,14 +478,13 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
         __builtin_amdgcn_wave_barrier();
         const bf16x8 pa = *(const bf16x8*)(pw + col * PSTR + (8 * g) * 2);
         // ---- O += P c ----
-        const int q4 = col >> 2, p4 = SWZ ? (col & 3) ^ ((g & 1) << 1) : col & 3;  // rows 8.. of 16: halves swapped
+        const int q4 = col >> 2, p4 = col & 3;
         const char* vlo = c_lds + (8 * g + q4) * CSTR + 8 * p4;
         const char* vhi = c_lds + (8 * g + 4 + q4) * CSTR + 8 * p4;
 #pragma unroll
         for (int nt = 0; nt < RV * 2; ++nt) {
-            const int gr = SWZ ? nt ^ ((g & 1) << 2) : nt;  // 32-byte granule of rows 8g.. (XOR 8 on pieces = 4 on granules; the XOR 1 is in p4)
-            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MX_LDS s16x4*)(vlo + gr * 32));
-            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MX_LDS s16x4*)(vhi + gr * 32));
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MX_LDS s16x4*)(vlo + nt * 32));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MX_LDS s16x4*)(vhi + nt * 32));
             // whole-vector reinterpretation (element-wise bit casts of the transposed read have been miscompiled)
             const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
             const u32x4 w4 = {l2[0], l2[1], h2[0], h2[1]};
@@ -535,7 +528,7 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
 template <int RV, int NW>
 int launch_mfma(const AttnArgs& a, int n_rows, hipStream_t st) {
     constexpr int RP = RV * 32, BM = NW * 16;
-    constexpr size_t lds = (size_t)32 * (RP * 2 + (RV % 4 == 0 ? 32 : 16)) + (size_t)NW * 16 * (32 * 2 + 16);
+    constexpr size_t lds = (size_t)32 * (RP * 2 + 16) + (size_t)NW * 16 * (32 * 2 + 16);
     static_assert(lds <= 64 * 1024, "tile does not fit the LDS of a workgroup");
     const int tiles = a.cu_q ? (n_rows * a.H + BM - 1) / BM + a.n_seqs : a.n_seqs * ((a.H + BM - 1) / BM);
     dim3 grid(tiles, a.parts);
