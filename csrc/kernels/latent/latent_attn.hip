@@ -296,13 +296,20 @@ MX_DEV float group_sum16(float v) {
     return v + __shfl_xor(v, 8, 64);
 }
 
-template <int RV, int NW>
-__global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
-    constexpr int RP = RV * 32, KT = 32, CSTR = RP * 2 + 16, PSTR = KT * 2 + 16, BM = NW * 16, NTH = NW * 64;
+// RS = 2 splits the rank between two waves of a row tile: both compute the tile's full scores and softmax (no
+// exchange, no extra barrier), each accumulates and writes one half of the output columns. Half the accumulators per
+// wave let two waves share a SIMD at the widest ranks, which is what hides the latencies between a tile's steps.
+template <int RV, int NW, int RS>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(RS == 2 ? 2 : 1)))
+void latent_attn_mfma_kernel(AttnArgs a) {
+    constexpr int RP = RV * 32, KT = 32, CSTR = RP * 2 + 16, PSTR = KT * 2 + 16, NTH = NW * 64;
+    constexpr int BM = NW / RS * 16, NO = RV * 2 / RS;  // rows per workgroup, output column tiles per wave
+    static_assert(NW % RS == 0 && (RV * 2) % RS == 0, "rank split");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char* c_lds = smem;                                   // [KT][CSTR] bf16 latents of the tile
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, g = lane >> 4;
-    char* pw = smem + KT * CSTR + wave * 16 * PSTR;       // this wave's P [16][PSTR]
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, col = lane & 15, g = lane >> 4;
+    const int wave = wv / RS, half = wv % RS;  // row tile of this wave, and which part of the rank it accumulates
+    char* pw = smem + KT * CSTR + wv * 16 * PSTR;       // this wave's P [16][PSTR]
     const int H = a.H, R = a.R;
     const bf16_t* qa = (const bf16_t*)a.qa;
     const bf16_t* cache = (const bf16_t*)a.cache;
@@ -370,14 +377,14 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
         trow_i[i] = (long)a.row_base + crow0 + t;
     }
     float mrow[4], lrow[4];
-    f32x4 oacc[RV * 2];
+    f32x4 oacc[NO];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         mrow[i] = -INFINITY;
         lrow[i] = 0.f;
     }
 #pragma unroll
-    for (int nt = 0; nt < RV * 2; ++nt) oacc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < NO; ++nt) oacc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
     const int* btr = a.bt + (long)seq * a.bt_stride;
     const float scale = a.scale;
     const bool wave_active = g0 + 16 * wave < nrows;
@@ -386,7 +393,7 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
     // current tile's products and stay in registers meanwhile (all of a tile when NTH * UB covers it); the rest
     // is loaded UB pieces at a time once the tile's turn has come.
     const int bs_shift = (a.bs & (a.bs - 1)) == 0 ? __builtin_ctz(a.bs) : -1;
-    constexpr int CPK = RP / 8, TOTAL = KT * CPK, UB = (NW == 1 && RV > 8) ? 4 : 8;  // registers are full at RV 16
+    constexpr int CPK = RP / 8, TOTAL = KT * CPK, UB = (NW == 1 && RV > 8) || NW == 8 || (RS == 2 && RV > 12) ? 4 : 8;  // register room at the widest ranks
     u32x4 pre[UB];
     auto fetch = [&](int k0, int base, u32x4* v) {
 #pragma unroll
@@ -464,7 +471,7 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
         const bool moved = alpha[0] != 1.f || alpha[1] != 1.f || alpha[2] != 1.f || alpha[3] != 1.f;
         if (__builtin_amdgcn_ballot_w64(moved) != 0) {
 #pragma unroll
-            for (int nt = 0; nt < RV * 2; ++nt)
+            for (int nt = 0; nt < NO; ++nt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) oacc[nt][i] *= alpha[i];
         }
@@ -479,10 +486,10 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
         const bf16x8 pa = *(const bf16x8*)(pw + col * PSTR + (8 * g) * 2);
         // ---- O += P c ----
         const int q4 = col >> 2, p4 = col & 3;
-        const char* vlo = c_lds + (8 * g + q4) * CSTR + 8 * p4;
-        const char* vhi = c_lds + (8 * g + 4 + q4) * CSTR + 8 * p4;
+        const char* vlo = c_lds + (8 * g + q4) * CSTR + 8 * p4 + half * NO * 32;
+        const char* vhi = c_lds + (8 * g + 4 + q4) * CSTR + 8 * p4 + half * NO * 32;
 #pragma unroll
-        for (int nt = 0; nt < RV * 2; ++nt) {
+        for (int nt = 0; nt < NO; ++nt) {
             const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MX_LDS s16x4*)(vlo + nt * 32));
             const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MX_LDS s16x4*)(vhi + nt * 32));
             // whole-vector reinterpretation (element-wise bit casts of the transposed read have been miscompiled)
@@ -499,13 +506,13 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
         for (int i = 0; i < 4; ++i) {
             if (!valid_i[i]) continue;
             const long prow = ((long)seq * H + head_i[i]) * a.parts + part;
-            if (col == 0) {
+            if (col == 0 && half == 0) {
                 a.part_ml[prow * 2] = mrow[i];
                 a.part_ml[prow * 2 + 1] = lrow[i];
             }
 #pragma unroll
-            for (int nt = 0; nt < RV * 2; ++nt) {
-                const int r = 16 * nt + col;
+            for (int nt = 0; nt < NO; ++nt) {
+                const int r = 16 * (half * NO + nt) + col;
                 if (r < R) a.part_o[prow * R + r] = oacc[nt][i];
             }
         }
@@ -518,31 +525,38 @@ __global__ __launch_bounds__(NW * 64) void latent_attn_mfma_kernel(AttnArgs a) {
         const float inv = lrow[i] > 0.f ? 1.f / lrow[i] : 0.f;
         bf16_t* orow = out + trow_i[i] * a.os_t + (long)head_i[i] * a.os_h;
 #pragma unroll
-        for (int nt = 0; nt < RV * 2; ++nt) {
-            const int r = 16 * nt + col;
+        for (int nt = 0; nt < NO; ++nt) {
+            const int r = 16 * (half * NO + nt) + col;
             if (r < R) orow[r] = f32_to_bf16(oacc[nt][i] * inv);
         }
     }
 }
 
-template <int RV, int NW>
+template <int RV, int NW, int RS>
 int launch_mfma(const AttnArgs& a, int n_rows, hipStream_t st) {
-    constexpr int RP = RV * 32, BM = NW * 16;
+    constexpr int RP = RV * 32, BM = NW / RS * 16;
     constexpr size_t lds = (size_t)32 * (RP * 2 + 16) + (size_t)NW * 16 * (32 * 2 + 16);
     static_assert(lds <= 64 * 1024, "tile does not fit the LDS of a workgroup");
     const int tiles = a.cu_q ? (n_rows * a.H + BM - 1) / BM + a.n_seqs : a.n_seqs * ((a.H + BM - 1) / BM);
     dim3 grid(tiles, a.parts);
-    latent_attn_mfma_kernel<RV, NW><<<grid, NW * 64, lds, st>>>(a);
+    latent_attn_mfma_kernel<RV, NW, RS><<<grid, NW * 64, lds, st>>>(a);
     return (int)hipGetLastError();
 }
 
 template <int RV>
 int dispatch_mfma_nw(const AttnArgs& a, int n_rows, hipStream_t st) {
-    // prompt chunks fill four waves. A decode row set is one token's H heads: up to 32 of them take two waves
-    // (the second only helps to fetch the key tiles when H <= 16), which leaves room for a second workgroup on the
-    // CU at the register budget of the widest ranks; more heads take four
-    if (!a.cu_q && a.H <= 32) return launch_mfma<RV, 2>(a, n_rows, st);
-    return launch_mfma<RV, 4>(a, n_rows, st);
+    // Row tiles per workgroup: prompt chunks four. A decode row set is one token's H heads: up to 16 take one row
+    // tile, up to 32 two, more four. Ranks of 256 and more split each row tile between two waves (RS 2); narrower
+    // ones keep one wave per row tile, with a second wave that only helps to fetch when there is a single row tile.
+    const int rows = a.cu_q ? 64 : a.H;
+    if constexpr (RV >= 8 && RV % 2 == 0) {
+        if (rows <= 16) return launch_mfma<RV, 2, 2>(a, n_rows, st);
+        if (rows <= 32) return launch_mfma<RV, 4, 2>(a, n_rows, st);
+        return launch_mfma<RV, 8, 2>(a, n_rows, st);
+    } else {
+        if (rows <= 32) return launch_mfma<RV, 2, 1>(a, n_rows, st);
+        return launch_mfma<RV, 4, 1>(a, n_rows, st);
+    }
 }
 
 int dispatch_mfma(const AttnArgs& a, int n_rows, hipStream_t st) {
