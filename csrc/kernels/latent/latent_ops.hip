@@ -43,6 +43,8 @@ MX_DEV void st_elem(void* p, long i, float v) {
     else ((float*)p)[i] = v;
 }
 
+constexpr int RC = 16;  // rows of up to NT * RC numbers are read once and kept in registers
+
 template <bool B16>
 __global__ __launch_bounds__(NT) void embed_norm_kernel(const void* table, int V, const int* tokens, const float* g,
                                                         float eps, float* out, int ldo, int C) {
@@ -51,18 +53,35 @@ __global__ __launch_bounds__(NT) void embed_norm_kernel(const void* table, int V
     int tok = tokens[t];
     if (tok < 0 || tok >= V) tok = 0;
     const long base = (long)tok * C;
+    const bool cached = C <= NT * RC;
+    float keep[RC];
     float ss = 0.f;
-    for (int c = threadIdx.x; c < C; c += NT) {
-        const float v = ld_elem<B16>(table, base + c);
-        ss += v * v;
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {  // clamped addresses: straight-line loads, all in flight together
+            const int c = threadIdx.x + k * NT;
+            const float v = ld_elem<B16>(table, base + min(c, C - 1));
+            keep[k] = c < C ? v : 0.f;
+            ss += keep[k] * keep[k];
+        }
+    } else {
+        for (int c = threadIdx.x; c < C; c += NT) {
+            const float v = ld_elem<B16>(table, base + c);
+            ss += v * v;
+        }
     }
     ss = block_sum(ss, red);
     const float sc = g[0] / sqrtf(ss / (float)C + eps);
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {
+            const int c = threadIdx.x + k * NT;
+            if (c < C) out[(long)t * ldo + c] = keep[k] * sc;
+        }
+        return;
+    }
     for (int c = threadIdx.x; c < C; c += NT) out[(long)t * ldo + c] = ld_elem<B16>(table, base + c) * sc;
 }
-
-// rows of up to NT * RC numbers are read once and kept in registers between the statistics and the output pass
-constexpr int RC = 16;
 
 __global__ __launch_bounds__(NT) void scalar_norm_kernel(const float* x, int ldx, const int* rows, const float* g,
                                                          float eps, float* o32, int ld32, bf16_t* o16, int ld16,
@@ -75,9 +94,10 @@ __global__ __launch_bounds__(NT) void scalar_norm_kernel(const float* x, int ldx
     float ss = 0.f;
     if (cached) {
 #pragma unroll
-        for (int k = 0; k < RC; ++k) {
+        for (int k = 0; k < RC; ++k) {  // clamped addresses: straight-line loads, all in flight together
             const int c = threadIdx.x + k * NT;
-            keep[k] = c < C ? xr[c] : 0.f;
+            const float v = xr[min(c, C - 1)];
+            keep[k] = c < C ? v : 0.f;
             ss += keep[k] * keep[k];
         }
     } else {
@@ -120,11 +140,18 @@ __global__ __launch_bounds__(NT) void gated_norm_add_kernel(float* x, int ldx, c
     float ss = 0.f;
     if (cached) {
         // every load of the row (the residual too) is issued before the statistics: one memory round trip
+        float yv[RC], gv[RC];
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {  // clamped addresses: straight-line loads, all in flight together
+            const int c = min(threadIdx.x + k * NT, C - 1);
+            xin[k] = x[(long)i * ldx + c];
+            yv[k] = yr[c];
+            gv[k] = gr[c] + (gb ? gb[c] : 0.f);
+        }
 #pragma unroll
         for (int k = 0; k < RC; ++k) {
             const int c = threadIdx.x + k * NT;
-            xin[k] = c < C ? x[(long)i * ldx + c] : 0.f;
-            keep[k] = c < C ? yr[c] * sigmoidf_(gr[c] + (gb ? gb[c] : 0.f)) : 0.f;
+            keep[k] = c < C ? yv[k] * sigmoidf_(gv[k]) : 0.f;
             ss += keep[k] * keep[k];
         }
     } else {
