@@ -127,11 +127,14 @@ __global__ __launch_bounds__(NT) void scalar_norm_kernel(const float* x, int ldx
     }
 }
 
-// x += g * unit_rms(z), z = y * sigmoid(gate_pre + gate_bias)
+// x += g * unit_rms(z), z = y * sigmoid(gate_pre + gate_bias); then, when gn is given, the NEXT norm of the updated
+// row in the same pass: n = gn * unit_rms(x) written as fp32 and / or bf16 (the row is still in registers)
 __global__ __launch_bounds__(NT) void gated_norm_add_kernel(float* x, int ldx, const float* y, int ldy,
                                                             const float* gp, int ldg, const float* gb, const float* g,
-                                                            float eps, int C) {
+                                                            float eps, int C, const float* gn, float* n32, int ldn32,
+                                                            bf16_t* n16, int ldn16) {
     __shared__ float red[NT / 64];
+    __shared__ float red2[NT / 64];
     const int i = blockIdx.x;
     const float* yr = y + (long)i * ldy;
     const float* gr = gp + (long)i * ldg;
@@ -162,16 +165,42 @@ __global__ __launch_bounds__(NT) void gated_norm_add_kernel(float* x, int ldx, c
     }
     ss = block_sum(ss, red);
     const float sc = g[0] / sqrtf(ss / (float)C + eps);
+    float s2 = 0.f;
     if (cached) {
 #pragma unroll
         for (int k = 0; k < RC; ++k) {
             const int c = threadIdx.x + k * NT;
-            if (c < C) x[(long)i * ldx + c] = xin[k] + keep[k] * sc;
+            xin[k] = c < C ? xin[k] + keep[k] * sc : 0.f;
+            if (c < C) x[(long)i * ldx + c] = xin[k];
+            s2 += xin[k] * xin[k];
+        }
+    } else {
+        for (int c = threadIdx.x; c < C; c += NT) {
+            const float v = x[(long)i * ldx + c] + yr[c] * sigmoidf_(gr[c] + (gb ? gb[c] : 0.f)) * sc;
+            x[(long)i * ldx + c] = v;
+            s2 += v * v;
+        }
+    }
+    if (gn == nullptr) return;
+    s2 = block_sum(s2, red2);
+    const float sn = gn[0] / sqrtf(s2 / (float)C + eps);
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {
+            const int c = threadIdx.x + k * NT;
+            if (c < C) {
+                const float v = xin[k] * sn;
+                if (n32) n32[(long)i * ldn32 + c] = v;
+                if (n16) n16[(long)i * ldn16 + c] = f32_to_bf16(v);
+            }
         }
         return;
     }
-    for (int c = threadIdx.x; c < C; c += NT)
-        x[(long)i * ldx + c] += yr[c] * sigmoidf_(gr[c] + (gb ? gb[c] : 0.f)) * sc;
+    for (int c = threadIdx.x; c < C; c += NT) {  // the thread re-reads what it wrote itself
+        const float v = x[(long)i * ldx + c] * sn;
+        if (n32) n32[(long)i * ldn32 + c] = v;
+        if (n16) n16[(long)i * ldn16 + c] = f32_to_bf16(v);
+    }
 }
 
 template <bool B16>
@@ -305,10 +334,12 @@ extern "C" int mxl_scalar_norm(const float* x, int ldx, const int* rows, const f
 }
 
 extern "C" int mxl_gated_norm_add(float* x, int ldx, const float* y, int ldy, const float* gp, int ldg, const float* gb,
-                                  const float* g, float eps, int M, int C, hipStream_t st) {
+                                  const float* g, float eps, int M, int C, const float* gn, float* n32, int ldn32,
+                                  bf16_t* n16, int ldn16, hipStream_t st) {
     if (M <= 0) return 0;
     MXL_CHECK(x && y && gp && g && C > 0 && ldx >= C && ldy >= C && ldg >= C);
-    gated_norm_add_kernel<<<M, NT, 0, st>>>(x, ldx, y, ldy, gp, ldg, gb, g, eps, C);
+    MXL_CHECK(!gn || ((n32 || n16) && (!n32 || ldn32 >= C) && (!n16 || ldn16 >= C)));
+    gated_norm_add_kernel<<<M, NT, 0, st>>>(x, ldx, y, ldy, gp, ldg, gb, g, eps, C, gn, n32, ldn32, n16, ldn16);
     return (int)hipGetLastError();
 }
 

@@ -125,8 +125,8 @@ LATENT_SIGS = {
     "mxl_embed_norm": [P, I, I, P, P, F, P, I, I, I, P],
     # x, ldx, rows, g, eps, out32, ld32, out16, ld16, M, C, stream
     "mxl_scalar_norm": [P, I, P, P, F, P, I, P, I, I, I, P],
-    # x, ldx, y, ldy, gate_pre, ldg, gate_bias, g, eps, M, C, stream
-    "mxl_gated_norm_add": [P, I, P, I, P, I, P, P, F, I, I, P],
+    # x, ldx, y, ldy, gate_pre, ldg, gate_bias, g, eps, M, C, g_next, next32, ld32, next16, ld16, stream
+    "mxl_gated_norm_add": [P, I, P, I, P, I, P, P, F, I, I, P, P, I, P, I, P],
     # u, ldu, out, ldo, is16, M, F, stream
     "mxl_relu2": [P, I, P, I, I, I, I, P],
     # h, ldh, w, taps, tails, state, positions, n_dec, pf_cu, n_pf, out, ldo, is16, T, C, stream

@@ -329,6 +329,7 @@ class VosotarModel:
         hm = ws.hm[:T]
         gate = ws.gate[:T * C].view(T, C)
         y = ws.y[:T * C].view(T, C)
+        normed = False  # h32 / hin already hold this layer's first norm
         for li, L in enumerate(cfg.layers):
             if fb.stop_layer is not None and li >= fb.stop_layer:
                 break
@@ -337,7 +338,8 @@ class VosotarModel:
             H, d, dv, R, Rq = mx.heads, mx.dim, mx.vdim, mx.kv_rank, mx.q_rank
             lat, tails = cache.layer(li)
             # ---- mixer ----
-            LA.scalar_rmsnorm(x, W.n1, eps, out32=h32, out16=hin if b16 else None)
+            if not normed:  # (otherwise the previous layer's last gated add wrote this norm in its own pass)
+                LA.scalar_rmsnorm(x, W.n1, eps, out32=h32, out16=hin if b16 else None)
             W.rg1.into(hin, gate)
             LA.tap_conv(h32, W.canon, tails, rag, hm)
             n_in = Rq + R + H
@@ -357,18 +359,28 @@ class VosotarModel:
             att = ws.att[:T * H * dv].view(T, H * dv)
             LA.head_gate_pack(ov, y_in[:, Rq + R:], att)
             W.o.into(att, y)
-            LA.gated_norm_add(x, y, gate, W.n1b, eps, W.rg1_b)
-            # ---- feed-forward ----
+            # the norm that follows a gated add (this layer's feed-forward norm, or the next layer's first norm) is
+            # written by the add's own pass
+            nxt = cfg.layers[li + 1] if li + 1 < len(cfg.layers) and (fb.stop_layer is None or li + 1 < fb.stop_layer) \
+                else None
+            Wn = self.weights[nxt.weights_of if nxt.weights_of is not None else li + 1] if nxt is not None else None
             if L.ff is None:
+                LA.gated_norm_add(x, y, gate, W.n1b, eps, W.rg1_b, next_g=Wn.n1 if Wn is not None else None,
+                                  next32=h32, next16=hin if b16 else None)
+                normed = Wn is not None
                 continue
+            LA.gated_norm_add(x, y, gate, W.n1b, eps, W.rg1_b, next_g=W.n2, next32=None if b16 else h32,
+                              next16=hin if b16 else None)
+            # ---- feed-forward ----
             F_ = L.ff
-            LA.scalar_rmsnorm(x, W.n2, eps, out32=None if b16 else h32, out16=hin if b16 else None)
             u = ws.u[:T * (F_ + C)].view(T, F_ + C)
             W.up_rg2.into(hin, u)
             act = ws.act[:T * F_].view(T, F_)
             LA.relu2(u[:, :F_], act)
             W.down.into(act, y)
-            LA.gated_norm_add(x, y, u[:, F_:], W.n2b, eps, W.rg2_b)
+            LA.gated_norm_add(x, y, u[:, F_:], W.n2b, eps, W.rg2_b, next_g=Wn.n1 if Wn is not None else None,
+                              next32=h32, next16=hin if b16 else None)
+            normed = Wn is not None
         if fb.stop_layer is not None:
             return x
         # ---- head ----

@@ -91,9 +91,11 @@ def scalar_rmsnorm(x: torch.Tensor, g: torch.Tensor, eps: float, out32: torch.Te
 
 
 def gated_norm_add(x: torch.Tensor, y: torch.Tensor, gate_pre: torch.Tensor, g: torch.Tensor, eps: float,
-                   gate_bias: torch.Tensor | None = None):
+                   gate_bias: torch.Tensor | None = None, next_g: torch.Tensor | None = None,
+                   next32: torch.Tensor | None = None, next16: torch.Tensor | None = None):
     """x += unit_rms(y * sigmoid(gate_pre + gate_bias)) * g on fp32 rows [M, C]; gate_pre may be a column slice,
-    gate_bias is fp32 [C]."""
+    gate_bias is fp32 [C]. With `next_g` the same pass also writes the following scalar-gain norm of the updated
+    rows, next_g * unit_rms(x), as fp32 (`next32`) and / or bf16 (`next16`)."""
     M, C = y.shape
     if M == 0:
         return x
@@ -101,9 +103,13 @@ def gated_norm_add(x: torch.Tensor, y: torch.Tensor, gate_pre: torch.Tensor, g: 
         gp = gate_pre.float() + gate_bias if gate_bias is not None else gate_pre.float()
         z = y.float() * torch.sigmoid(gp)
         x.add_(z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps) * g.float())
+        if next_g is not None:
+            scalar_rmsnorm(x, next_g, eps, out32=next32, out16=next16)
         return x
     N.kcall("mxl_gated_norm_add", x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0), gate_pre.data_ptr(),
-            gate_pre.stride(0), N.ptr(gate_bias), g.data_ptr(), float(eps), M, C, N.stream_ptr())
+            gate_pre.stride(0), N.ptr(gate_bias), g.data_ptr(), float(eps), M, C, N.ptr(next_g), N.ptr(next32),
+            next32.stride(0) if next32 is not None else 0, N.ptr(next16),
+            next16.stride(0) if next16 is not None else 0, N.stream_ptr())
     return x
 
 

@@ -116,11 +116,24 @@ def test_norms_gate_and_activation(dev):
     LA.gated_norm_add(res, y.to(dev), wide.to(dev)[:, 9:], gain.to(dev), eps, bias.to(dev))
     close(res.cpu(), x.double() + O.scalar_norm(y.double() * torch.sigmoid(wide.double()[:, 9:] + bias.double()),
                                                 gain, eps), 1e-5)
+    # the following norm written by the same pass
+    res, n32 = x.clone().to(dev), torch.empty(M, C, device=dev)
+    n16 = torch.empty(M, C, device=dev, dtype=torch.bfloat16)
+    g2n = torch.tensor([0.6])
+    LA.gated_norm_add(res, y.to(dev), wide.to(dev)[:, 9:], gain.to(dev), eps, bias.to(dev), next_g=g2n.to(dev),
+                      next32=n32, next16=n16)
+    upd = x.double() + O.scalar_norm(y.double() * torch.sigmoid(wide.double()[:, 9:] + bias.double()), gain, eps)
+    close(res.cpu(), upd, 1e-5)
+    close(n32.cpu(), O.scalar_norm(upd, g2n, eps), 1e-5)
+    close(n16.float().cpu(), O.scalar_norm(upd, g2n, eps), 1e-2)
     for C2 in (4100, 5000):  # rows wider than the kernels keep in registers
         x2, y2, g2 = (torch.randn(3, C2, generator=g) for _ in range(3))
         r2, n2 = x2.clone().to(dev), torch.empty(3, C2, device=dev)
-        LA.gated_norm_add(r2, y2.to(dev), g2.to(dev), gain.to(dev), eps)
-        close(r2.cpu(), x2.double() + O.scalar_norm(y2.double() * torch.sigmoid(g2.double()), gain, eps), 1e-5)
+        w32 = torch.empty(3, C2, device=dev)
+        LA.gated_norm_add(r2, y2.to(dev), g2.to(dev), gain.to(dev), eps, next_g=g2n.to(dev), next32=w32)
+        u2 = x2.double() + O.scalar_norm(y2.double() * torch.sigmoid(g2.double()), gain, eps)
+        close(r2.cpu(), u2, 1e-5)
+        close(w32.cpu(), O.scalar_norm(u2, g2n, eps), 1e-5)
         LA.scalar_rmsnorm(x2.to(dev), gain.to(dev), eps, out32=n2)
         close(n2.cpu(), O.scalar_norm(x2.double(), gain, eps), 1e-5)
     # squared relu on a column slice
