@@ -345,9 +345,8 @@ extern "C" int mxl_gated_norm_add(float* x, int ldx, const float* y, int ldy, co
 
 extern "C" int mxl_relu2(const float* u, int ldu, void* out, int ldo, int is16, int M, int F, hipStream_t st) {
     if (M <= 0 || F <= 0) return 0;
-    MXL_CHECK(u && out && ldu >= F && ldo >= F && M <= 65535 * 64);
+    MXL_CHECK(u && out && ldu >= F && ldo >= F && M <= 65535);  // rows ride on grid.y
     dim3 grid(min((F + NT - 1) / NT, 64), M);
-    MXL_CHECK(M <= 65535);
     if (is16) relu2_kernel<true><<<grid, NT, 0, st>>>(u, ldu, out, ldo, F);
     else relu2_kernel<false><<<grid, NT, 0, st>>>(u, ldu, out, ldo, F);
     return (int)hipGetLastError();

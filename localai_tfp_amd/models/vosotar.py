@@ -29,7 +29,6 @@ import json
 import os
 from dataclasses import dataclass, field
 
-import numpy as np
 import torch
 
 from ..ops import latent as LA

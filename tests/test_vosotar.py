@@ -8,7 +8,6 @@ import json
 import math
 import os
 import subprocess
-import sys
 
 import numpy as np
 import pytest
