@@ -380,10 +380,11 @@ class LLMEngine:
             c.block_size = c.max_model_len
             c.enable_prefix_cache = False
             draft = None
-        # latent-cache models (models/vosotar.py): a paged pool of per-token latents, addressed like K / V blocks, plus
-        # one state slot per live sequence (SlotPool) for rows carried between steps. A cached block does not hold
-        # that carried state, so blocks are not shared between requests; no drafts, no TP
-        self.latent = getattr(model, "cache_kind", "") == "latent"
+        # paged-pool-plus-state models: a paged pool addressed like K / V blocks (per-token latents, models/vosotar.py;
+        # keys and values of the attention layers of a hybrid decoder, models/vugotar.py) plus one state slot per live
+        # sequence (SlotPool) for what is carried between steps (convolution tails, recurrent states). A cached block
+        # does not hold that carried state, so blocks are not shared between requests; no drafts, no TP
+        self.latent = getattr(model, "cache_kind", "") in ("latent", "hybrid")
         self.state_slots = None
         self._replay: dict = {}
         if self.latent:
@@ -408,8 +409,8 @@ class LLMEngine:
             nb = c.max_num_seqs + 1
             self.kv = model.make_state_cache(nb, c.block_size)
         elif self.latent:
-            ranks = model.cache_ranks()
-            nb = c.num_blocks or LatentCache.auto_num_blocks(ranks, c.block_size, self.device, frac,
+            # the model says how many pool numbers one token takes in each of its cached layers
+            nb = c.num_blocks or LatentCache.auto_num_blocks(model.cache_ranks(), c.block_size, self.device, frac,
                                                              dtype_bytes=model.dtype.itemsize)
             self.kv = model.make_cache(nb, c.block_size, c.max_num_seqs)
             self.state_slots = SlotPool(c.max_num_seqs)

@@ -206,6 +206,40 @@ class LatentCache:
         return max(n, 16)
 
 
+class HybridCache:
+    """Cache of decoders that mix paged attention with recurrent layers (ops/hybrid.py). Every layer RUN (a layer
+    that is looped counts once per pass) owns what its mixers need:
+
+    * `kv[i]`: (keys [num_blocks, block_size, kv_heads * dim], values [.., kv_heads * vdim]) in bf16 or fp32,
+      token-major so one append writes one contiguous row, addressed by the block tables and flat slots of the block
+      manager; None for runs without attention;
+    * `state[i]`: fp32 [state_slots, heads, N, P] recurrent state, None for runs without a recurrence;
+    * `tails[i]`: fp32 [state_slots, taps - 1, channels] last inputs of the run's causal convolution, or None.
+
+    `spec` lists per run a dict with the optional keys "kv": (key row, value row), "state": (heads, N, P),
+    "tails": (taps - 1, channels). State slots are handed out per live sequence by `SlotPool`."""
+
+    def __init__(self, spec, num_blocks: int, block_size: int, device, dtype=torch.bfloat16, state_slots: int = 0):
+        self.n_layers, self.num_blocks, self.block_size = len(spec), num_blocks, block_size
+        self.state_slots = state_slots
+        S = max(1, state_slots)
+        f32 = dict(dtype=torch.float32, device=device)
+        self.kv, self.state, self.tails = [], [], []
+        for e in spec:
+            kv, st, tl = e.get("kv"), e.get("state"), e.get("tails")
+            self.kv.append(None if kv is None else
+                           (torch.zeros((num_blocks, block_size, int(kv[0])), dtype=dtype, device=device),
+                            torch.zeros((num_blocks, block_size, int(kv[1])), dtype=dtype, device=device)))
+            self.state.append(None if st is None else torch.zeros((S, *[int(x) for x in st]), **f32))
+            self.tails.append(None if tl is None else torch.zeros((S, max(1, int(tl[0])), int(tl[1])), **f32))
+
+    def layer(self, i: int):
+        return self.kv[i], self.state[i], self.tails[i]
+
+    def state_bytes_per_seq(self) -> int:
+        return int(sum(t[0].numel() * 4 for t in self.state + self.tails if t is not None))
+
+
 class SlotPool:
     """State slots of live sequences: a free list of `n` slots keyed by request id. A sequence takes a slot with
     its first scheduled tokens and keeps it until it finishes, is aborted or is preempted (its state is then

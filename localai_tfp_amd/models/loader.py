@@ -148,25 +148,37 @@ def _apply_overrides(cfg: LlamaConfig, ov: dict):
         cfg.ctx_train = max(cfg.ctx_train, int(ov["context_size"])) if ov.get("extend_context") else cfg.ctx_train
 
 
-def _load_latent(model: str, device, tp_size: int, ov: dict):
-    """Latent-attention decoders (models/vosotar.py): a directory whose config.json names the Vosotar architecture,
-    or `synthetic:vosotar-*` random weights. `overrides["dtype"]`: torch.bfloat16 (default on GPU) | torch.float32.
-    None for everything else."""
+def _state_families():
+    """Decoder families served from a paged pool plus per-sequence state slots, chosen by config.json's
+    `architecture`: name -> (module, model class name, config maker for `synthetic:<key>`)."""
     from . import vosotar as VO
+    from . import vugotar as VU
+    return {"vosotar": (VO, VO.VosotarModel, VO.is_vosotar_dir), "vugotar": (VU, VU.VugotarModel, VU.is_vugotar_dir)}
+
+
+def _load_latent(model: str, device, tp_size: int, ov: dict):
+    """Latent-attention decoders (models/vosotar.py) and hybrid attention / recurrent decoders (models/vugotar.py): a
+    directory whose config.json names the architecture, or `synthetic:vosotar-*` / `synthetic:vugotar-*` random
+    weights. `overrides["dtype"]`: torch.bfloat16 (default on GPU) | torch.float32. None for everything else."""
     from ..tokenizer import ByteTokenizer
-    synth = model.startswith("synthetic:vosotar")
-    if not synth and not VO.is_vosotar_dir(model):
+    fam = None
+    for key, (mod, klass, is_dir) in _state_families().items():
+        if model.startswith("synthetic:" + key) or (not model.startswith("synthetic:") and is_dir(model)):
+            fam = (key, mod, klass)
+            break
+    if fam is None:
         return None
+    key, mod, klass = fam
     if tp_size > 1:
-        raise ValueError("tensor parallelism is not supported for Vosotar models")
+        raise ValueError(f"tensor parallelism is not supported for {mod.ARCH} models")
     if ov.get("lora"):
-        raise NotImplementedError("LoRA adapters are not supported for Vosotar models")
-    if synth:
-        key = model.split(":", 1)[1]
-        cfg = VO.make_config(name=key, **VO.SYNTHETIC[key])
-        m = VO.VosotarModel.load(cfg, VO.synthetic_source(cfg, seed=1), device, ov.get("dtype"))
+        raise NotImplementedError(f"LoRA adapters are not supported for {mod.ARCH} models")
+    if model.startswith("synthetic:"):
+        name = model.split(":", 1)[1]
+        cfg = mod.make_config(name=name, **mod.SYNTHETIC[name])
+        m = klass.load(cfg, mod.synthetic_source(cfg, seed=1), device, ov.get("dtype"))
         return m, ByteTokenizer(cfg.vocab), cfg, {}
-    cfg, get = VO.dir_source(model)
+    cfg, get = mod.dir_source(model)
     tok = ByteTokenizer(cfg.vocab)
     if os.path.isfile(os.path.join(model, "tokenizer.json")):
         try:
@@ -174,7 +186,7 @@ def _load_latent(model: str, device, tp_size: int, ov: dict):
             tok = from_hf_dir(model)
         except Exception as ex:
             log.warning("no usable tokenizer in %s (%s); byte-level fallback", model, ex)
-    return VO.VosotarModel.load(cfg, get, device, ov.get("dtype")), tok, cfg, {}
+    return klass.load(cfg, get, device, ov.get("dtype")), tok, cfg, {}
 
 
 RECURRENT_ARCHS = {"mamba", "rwkv6"}

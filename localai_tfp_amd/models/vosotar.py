@@ -429,11 +429,9 @@ def is_vosotar_dir(path: str) -> bool:
         return False
 
 
-def dir_source(model_dir: str):
-    """(VosotarConfig, get) of a directory holding config.json and model.safetensors."""
+def tensor_getter(model_dir: str):
+    """get(name) -> tensor or None over every *.safetensors file of a directory (opened lazily, read by name)."""
     from safetensors import safe_open
-    with open(os.path.join(model_dir, "config.json")) as f:
-        cfg = VosotarConfig.from_json(json.load(f), os.path.basename(os.path.normpath(model_dir)))
     files = [os.path.join(model_dir, fn) for fn in sorted(os.listdir(model_dir)) if fn.endswith(".safetensors")]
     handles = [safe_open(fn, framework="pt") for fn in files]
     where = {k: h for h in handles for k in h.keys()}
@@ -441,7 +439,14 @@ def dir_source(model_dir: str):
     def get(name):
         h = where.get(name)
         return h.get_tensor(name) if h is not None else None
-    return cfg, get
+    return get
+
+
+def dir_source(model_dir: str):
+    """(VosotarConfig, get) of a directory holding config.json and model.safetensors."""
+    with open(os.path.join(model_dir, "config.json")) as f:
+        cfg = VosotarConfig.from_json(json.load(f), os.path.basename(os.path.normpath(model_dir)))
+    return cfg, tensor_getter(model_dir)
 
 
 def synthetic_source(cfg: VosotarConfig, seed: int = 0):

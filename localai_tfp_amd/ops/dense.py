@@ -83,6 +83,11 @@ class Dense:
 
     def acc(self, x: torch.Tensor, acc: torch.Tensor) -> torch.Tensor:
         """acc (fp32) += x W^T + b — the residual add fused as GEMM beta = 1."""
+        if x.dtype == torch.float32 and acc.is_contiguous():
+            if self.b32 is not None:
+                acc.add_(self.b32)
+            torch.addmm(acc, x, self.wt, out=acc)
+            return acc
         if x.dtype != torch.float32 and _fp32_out_ok(x.dtype) and acc.is_contiguous():
             if self.b32 is not None:
                 acc.add_(self.b32)

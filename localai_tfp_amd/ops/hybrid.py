@@ -1,0 +1,375 @@
+"""Ops of hybrid decoders that mix paged softmax attention with recurrent layers whose state is carried per sequence:
+
+* `embed_rows`, `offset_rmsnorm`: an fp32 residual from a 16-bit table; an RMS norm whose weight is stored around
+  an offset (x / rms * (offset + w));
+* `rope_norm_append`: rotary positions on neighbouring pairs of the first `rot_dims` numbers of each query / key
+  head, an optional unit-RMS norm of every head after the rotation, and the append of keys and values to paged pools;
+* `masked_attention`: causal attention over the paged pools whose visible range starts at a chunk border
+  (`chunk`), `window` keys back, or at position 0, with an optional sink (one extra term exp(0) in the softmax
+  denominator that carries no value);
+* `causal_conv`: a per-channel causal convolution over time (optional bias and SiLU) whose last taps-1 inputs are
+  carried per sequence;
+* `unit_norm_heads`, `scan_coefs`, `state_scan`: the pieces of a linear recurrence S <- a S + k u^T, o = S^T q per
+  head (S is [N, P], fp32, one per sequence and head). With `delta` the written value is u = c (v - S^T k) after
+  the decay (gated delta rule), otherwise u = c v with an optional skip D v on the output (state-space duality form);
+* `gated_group_norm`: unit-RMS norm over groups of columns, a weight, and a SiLU gate before or after the norm;
+* `glu`: silu(a + bias) * (b + bias) with an optional per-row, per-column-group factor (routing weights of experts
+  evaluated side by side, or the sigmoid gate of a shared expert);
+* `moe_route`: softmax over experts, the `top` largest, renormalised and scaled, as a dense [T, E] weight matrix.
+
+Every function runs the HIP kernels of csrc/kernels/hybrid/ on GPU tensors and a plain fp32 PyTorch form on CPU
+tensors (the plumbing path of GPU-less environments). Positions, angles, scores, softmax, norms, routing, decays,
+states and the residual are fp32 in both; 16-bit tensors appear only as GEMM operands and in the paged pools.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+from .. import _native as N
+from .latent import Ragged, _is16  # noqa: F401  (Ragged: the step layout shared with the latent ops)
+
+
+def _f32c(t: torch.Tensor, what: str):
+    if t.dtype != torch.float32 or t.stride(-1) != 1:
+        raise TypeError(f"{what}: fp32 rows with a contiguous last axis expected")
+
+
+# ------------------------------------------------------------------------------------------------ embedding, norm
+def embed_rows(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor, accumulate: bool = False):
+    """out[t] (=|+=) table[tokens[t]]; table fp32 or bf16 [V, C], out fp32 [T, C]."""
+    T, C = out.shape
+    if T == 0:
+        return out
+    if not out.is_cuda:
+        rows = table[tokens.long()].float()
+        out.add_(rows) if accumulate else out.copy_(rows)
+        return out
+    N.kcall("mxh_embed_rows", table.data_ptr(), _is16(table), table.shape[0], tokens.data_ptr(), out.data_ptr(),
+            out.stride(0), int(accumulate), T, C, N.stream_ptr())
+    return out
+
+
+def offset_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out32: torch.Tensor | None = None,
+                   out16: torch.Tensor | None = None, rows: torch.Tensor | None = None, offset: float = 1.0):
+    """y = x / sqrt(mean(x^2) + eps) * (offset + w) for fp32 rows, written as fp32 and / or bf16. `rows` (int32)
+    picks the rows of x to norm: output row i comes from x[rows[i]]."""
+    M = int(rows.numel()) if rows is not None else x.shape[0]
+    C = x.shape[1]
+    if M == 0:
+        return
+    if not x.is_cuda:
+        xs = x[rows.long()] if rows is not None else x
+        y = xs * torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + eps) * (offset + w.float())
+        if out32 is not None:
+            out32.copy_(y)
+        if out16 is not None:
+            out16.copy_(y)
+        return
+    _f32c(x, "offset_rmsnorm")
+    N.kcall("mxh_offset_norm", x.data_ptr(), x.stride(0), N.ptr(rows), w.data_ptr(), float(offset), float(eps),
+            N.ptr(out32), out32.stride(0) if out32 is not None else 0, N.ptr(out16),
+            out16.stride(0) if out16 is not None else 0, M, C, N.stream_ptr())
+
+
+# ------------------------------------------------------------------------------------------------ attention
+def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor, positions: torch.Tensor, H: int,
+                     G: int, dk: int, dv: int, rot_dims: int, rot_base: float, norm: bool, eps: float,
+                     q_out: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, slots: torch.Tensor):
+    """q_in [T, H*dk], k_in [T, G*dk], v_in [T, G*dv]: fp32 column slices of one projection output. Pair (2i, 2i+1)
+    of a head's first rot_dims numbers turns by positions[t] * rot_base^(-2i / rot_dims); with `norm` every query
+    and key head is then divided by its root mean square (eps inside the root). Queries go to q_out [T, H*dk]
+    (fp32 or bf16), keys and values into the paged pools kc [blocks, bs, G*dk] / vc [blocks, bs, G*dv] at flat slot
+    slots[t] (slot < 0: not stored)."""
+    T = q_in.shape[0]
+    if T == 0:
+        return
+    if rot_dims % 2 or rot_dims > dk:
+        raise ValueError("rope_norm_append: rot_dims is even and at most the head size")
+    if not q_in.is_cuda:
+        pos = positions.float()
+
+        def turn(x, n):
+            x = x.float().reshape(T, n, dk).clone()
+            if rot_dims:
+                i = torch.arange(rot_dims // 2, dtype=torch.float32)
+                a = pos[:, None] * torch.exp(i * (-2.0 / rot_dims * math.log(rot_base)))[None, :]
+                c, s = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+                u, v = x[..., 0:rot_dims:2].clone(), x[..., 1:rot_dims:2].clone()
+                x[..., 0:rot_dims:2] = u * c - v * s
+                x[..., 1:rot_dims:2] = v * c + u * s
+            if norm:
+                x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+            return x.reshape(T, n * dk)
+        q_out.copy_(turn(q_in, H))
+        ok = slots >= 0
+        kc.view(-1, G * dk)[slots[ok].long()] = turn(k_in, G)[ok].to(kc.dtype)
+        vc.view(-1, G * dv)[slots[ok].long()] = v_in.float()[ok].to(vc.dtype)
+        return
+    for t_ in (q_in, k_in, v_in):
+        _f32c(t_, "rope_norm_append")
+    if kc.dtype != vc.dtype or not kc.is_contiguous() or not vc.is_contiguous():
+        raise TypeError("rope_norm_append: contiguous key and value pools of one dtype")
+    N.kcall("mxh_rope_norm_append", q_in.data_ptr(), k_in.data_ptr(), v_in.data_ptr(), q_in.stride(0),
+            k_in.stride(0), v_in.stride(0), positions.data_ptr(), H, G, dk, dv, rot_dims, float(rot_base), int(norm),
+            float(eps), q_out.data_ptr(), q_out.stride(0), _is16(q_out), kc.data_ptr(), vc.data_ptr(), _is16(kc),
+            slots.data_ptr(), T, N.stream_ptr())
+
+
+def _attn_ref(q, kc, vc, table, ctx, pos0, H, G, dk, dv, scale, chunk, window, sink, out, out_scale):
+    bs = kc.shape[1]
+    nb = -(-ctx // bs)
+    k = kc[table[:nb].long()].reshape(nb * bs, G, dk)[:ctx].float()
+    v = vc[table[:nb].long()].reshape(nb * bs, G, dv)[:ctx].float()
+    n = q.shape[0]
+    qh = q.float().reshape(n, H, dk)
+    rep = H // G
+    s = torch.einsum("nhd,jhd->hnj", qh, k.repeat_interleave(rep, 1)) * scale
+    i = pos0 + torch.arange(n)[:, None]
+    j = torch.arange(ctx)[None, :]
+    lo = (i // chunk) * chunk if chunk else (i - window + 1).clamp(min=0) if window else torch.zeros_like(i)
+    vis = (j <= i) & (j >= lo)
+    s = s.masked_fill(~vis[None], float("-inf"))
+    m = s.max(-1, keepdim=True).values
+    if sink:
+        m = m.clamp(min=0.0)
+    e = torch.exp(s - m)
+    den = e.sum(-1, keepdim=True) + (torch.exp(-m) if sink else 0.0)
+    o = torch.einsum("hnj,jhe->nhe", e / den, v.repeat_interleave(rep, 1))
+    out.copy_((o.reshape(n, H * dv) * out_scale).to(out.dtype))
+
+
+def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: Ragged, H: int, G: int, dk: int, dv: int,
+                     scale: float, out: torch.Tensor, chunk: int = 0, window: int = 0, sink: bool = False,
+                     out_scale: float = 1.0):
+    """Causal attention of q [T, H*dk] over the paged pools (rope_norm_append's layout); query head h reads key /
+    value head h // (H / G). The row at position i sees j in [lo, i]: lo = (i // chunk) * chunk with `chunk`,
+    max(0, i - window + 1) with `window`, else 0. `sink` adds exp(0) to the softmax denominator. out [T, H*dv]
+    (may be a column slice; fp32 or bf16) receives out_scale times the result. q, pools and out share fp32 or bf16
+    operands; scores, softmax and the accumulators are fp32."""
+    T = q.shape[0]
+    if T == 0:
+        return out
+    if H % G:
+        raise ValueError("masked_attention: heads must be a multiple of kv heads")
+    nd = rag.n_dec
+    if not q.is_cuda:
+        if nd:
+            lens = rag.dec_lens.tolist()
+            for i in range(nd):
+                _attn_ref(q[i:i + 1], kc, vc, rag.dec_bt[i], lens[i], lens[i] - 1, H, G, dk, dv, scale, chunk, window,
+                          sink, out[i:i + 1], out_scale)
+        if rag.n_pf:
+            cu, ctx = rag.pf_cu.tolist(), rag.pf_ctx.tolist()
+            for k in range(rag.n_pf):
+                n = cu[k + 1] - cu[k]
+                if n:
+                    r0 = nd + cu[k]
+                    _attn_ref(q[r0:r0 + n], kc, vc, rag.pf_bt[k], ctx[k], ctx[k] - n, H, G, dk, dv, scale, chunk,
+                              window, sink, out[r0:r0 + n], out_scale)
+        return out
+    if q.dtype != kc.dtype or kc.dtype != vc.dtype or q.stride(1) != 1 or out.stride(1) != 1:
+        raise TypeError("masked_attention: queries and pools share one dtype, rows are contiguous")
+    bs = kc.shape[1]
+    st = N.stream_ptr()
+    common = (H, G, dk, dv, float(scale), int(chunk), int(window), int(sink), float(out_scale))
+    if nd:
+        N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
+                rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), None, rag.dec_lens.data_ptr(), nd, nd, 0,
+                out.data_ptr(), out.stride(0), _is16(out), *common, st)
+    if rag.n_pf:
+        N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
+                rag.pf_bt.data_ptr(), rag.pf_bt.stride(0), rag.pf_cu.data_ptr(), rag.pf_ctx.data_ptr(), rag.n_pf,
+                T - nd, nd, out.data_ptr(), out.stride(0), _is16(out), *common, st)
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ convolution
+def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, tails: torch.Tensor, rag: Ragged,
+                out: torch.Tensor, silu: bool = True):
+    """out_t = act(bias + sum_j w[:, j] * x_(t - taps + 1 + j)) per channel over each sequence's rows; the
+    sequence's previous taps-1 inputs are read from (and its newest written back to) `tails` [slots, taps-1, C]
+    fp32; a chunk that starts at position 0 reads zeros. x fp32 [T, C] (may be a column slice), w fp32 [C, taps],
+    out fp32 [T, C]. A state slot < 0 (padding rows) reads zeros and stores nothing."""
+    T, C = x.shape
+    taps = w.shape[1]
+    if T == 0:
+        return out
+    if not x.is_cuda:
+        st, pos = rag.state.tolist(), rag.positions.tolist()
+        for r0, n, si in rag.host_segments():
+            slot = st[si]
+            fresh = pos[r0] == 0 or slot < 0 or taps == 1
+            prev = torch.zeros(taps - 1, C) if fresh else tails[slot].clone()
+            full = torch.cat([prev, x[r0:r0 + n].float()], 0)
+            y = torch.zeros(n, C)
+            for j in range(taps):
+                y += w[:, j] * full[j:j + n]
+            if bias is not None:
+                y += bias
+            out[r0:r0 + n] = F.silu(y) if silu else y
+            if slot >= 0 and taps > 1:
+                tails[slot] = full[full.shape[0] - (taps - 1):]
+        return out
+    if taps > 16:
+        raise ValueError("causal_conv: at most 16 taps")
+    _f32c(x, "causal_conv")
+    _f32c(out, "causal_conv")
+    if tails.shape[1] != max(1, taps - 1) or tails.shape[2] != C or not tails.is_contiguous():
+        raise ValueError("causal_conv: tails are [slots, taps - 1, channels]")
+    N.kcall("mxh_causal_conv", x.data_ptr(), x.stride(0), w.data_ptr(), N.ptr(bias), taps, int(silu),
+            tails.data_ptr(), rag.state.data_ptr(), rag.positions.data_ptr(), rag.n_dec, N.ptr(rag.pf_cu), rag.n_pf,
+            out.data_ptr(), out.stride(0), T, C, N.stream_ptr())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ recurrences
+def unit_norm_heads(x: torch.Tensor, heads: int, dim: int, eps: float, scale: float = 1.0):
+    """In place on fp32 x [T, heads*dim]: every head becomes x / sqrt(sum(x^2) + eps) * scale."""
+    T = x.shape[0]
+    if T == 0:
+        return x
+    if not x.is_cuda:
+        v = x.reshape(T, heads, dim)
+        x.copy_((v * torch.rsqrt(v.pow(2).sum(-1, keepdim=True) + eps) * scale).reshape(T, heads * dim))
+        return x
+    _f32c(x, "unit_norm_heads")
+    N.kcall("mxh_unit_norm", x.data_ptr(), x.stride(0), heads, dim, float(eps), float(scale), T, N.stream_ptr())
+    return x
+
+
+def scan_coefs(a: torch.Tensor, b: torch.Tensor | None, A_log: torch.Tensor, dt_bias: torch.Tensor,
+               decay: torch.Tensor, coef: torch.Tensor):
+    """Per token and head: s = softplus(a + dt_bias), decay = exp(-exp(A_log) * s), coef = sigmoid(b) when b is
+    given, else s. a, b fp32 [T, H] column slices; decay, coef fp32 [T, H] contiguous."""
+    T, H = a.shape
+    if T == 0:
+        return
+    if not a.is_cuda:
+        s = F.softplus(a.float() + dt_bias, threshold=30.0)
+        decay.copy_(torch.exp(-torch.exp(A_log) * s))
+        coef.copy_(torch.sigmoid(b.float()) if b is not None else s)
+        return
+    N.kcall("mxh_scan_coefs", a.data_ptr(), a.stride(0), N.ptr(b), b.stride(0) if b is not None else 0,
+            A_log.data_ptr(), dt_bias.data_ptr(), decay.data_ptr(), coef.data_ptr(), T, H, N.stream_ptr())
+
+
+def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, coef: torch.Tensor,
+               skip: torch.Tensor | None, state: torch.Tensor, rag: Ragged, out: torch.Tensor, H: int, G: int, Nk: int,
+               P: int, delta: bool):
+    """Linear recurrence per sequence and head over the step's rows, in order:
+        S <- decay_t S;  u = coef_t (v_t - S^T k_t) if delta else coef_t v_t;  S <- S + k_t u^T;
+        o_t = S^T q_t (+ skip_h v_t)
+    k, q fp32 [T, G*Nk] (head h reads group h // (H / G)), v fp32 [T, H*P], decay / coef fp32 [T, H], out fp32
+    [T, H*P]; all may be column slices. state fp32 [slots, H, Nk, P] is read at the sequence's slot unless its first
+    row is at position 0 (then S starts at zero) and written back after its last row."""
+    T = k.shape[0]
+    if T == 0:
+        return out
+    if not k.is_cuda:
+        st, pos = rag.state.tolist(), rag.positions.tolist()
+        rep = H // G
+        for r0, n, si in rag.host_segments():
+            slot = st[si]
+            S = torch.zeros(H, Nk, P) if (pos[r0] == 0 or slot < 0) else state[slot].clone()
+            for t in range(r0, r0 + n):
+                kt = k[t].float().reshape(G, Nk).repeat_interleave(rep, 0)
+                qt = q[t].float().reshape(G, Nk).repeat_interleave(rep, 0)
+                vt = v[t].float().reshape(H, P)
+                S = S * decay[t][:, None, None]
+                u = coef[t][:, None] * ((vt - torch.einsum("hnp,hn->hp", S, kt)) if delta else vt)
+                S = S + kt[:, :, None] * u[:, None, :]
+                o = torch.einsum("hnp,hn->hp", S, qt)
+                if skip is not None:
+                    o = o + skip[:, None] * vt
+                out[t] = o.reshape(H * P)
+            if slot >= 0:
+                state[slot] = S
+        return out
+    for t_ in (k, q, v, out):
+        _f32c(t_, "state_scan")
+    if tuple(state.shape[1:]) != (H, Nk, P) or not state.is_contiguous() or not decay.is_contiguous() \
+            or not coef.is_contiguous() or H % G or Nk > 256:
+        raise ValueError("state_scan: state is [slots, H, N, P] with N <= 256, decay / coef contiguous [T, H]")
+    N.kcall("mxh_state_scan", k.data_ptr(), k.stride(0), q.data_ptr(), q.stride(0), v.data_ptr(), v.stride(0),
+            decay.data_ptr(), coef.data_ptr(), N.ptr(skip), state.data_ptr(), rag.state.data_ptr(),
+            rag.positions.data_ptr(), rag.n_dec, N.ptr(rag.pf_cu), rag.n_pf, out.data_ptr(), out.stride(0), H, G, Nk,
+            P, int(delta), N.stream_ptr())
+    return out
+
+
+def gated_group_norm(y: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, eps: float, group: int, out: torch.Tensor,
+                     gate_first: bool, out_scale: float = 1.0):
+    """Rows y [T, C] fp32 in groups of `group` columns, gate [T, C] fp32 (pre-activation), w fp32 whose length divides
+    C (column c uses w[c % len(w)]). gate_first: z = y * silu(gate), out = unit_rms_group(z) * w; otherwise
+    out = unit_rms_group(y) * w * silu(gate). out (fp32 or bf16, may be a column slice) gets out_scale times that."""
+    T, C = y.shape
+    if T == 0:
+        return out
+    if C % group or C % w.numel():
+        raise ValueError("gated_group_norm: group size and weight length divide the row")
+    if not y.is_cuda:
+        g = F.silu(gate.float())
+        z = (y.float() * g if gate_first else y.float()).reshape(T, C // group, group)
+        z = (z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, C) * w.float().repeat(C // w.numel())
+        out.copy_(((z if gate_first else z * g) * out_scale).to(out.dtype))
+        return out
+    _f32c(y, "gated_group_norm")
+    _f32c(gate, "gated_group_norm")
+    N.kcall("mxh_gated_group_norm", y.data_ptr(), y.stride(0), gate.data_ptr(), gate.stride(0), w.data_ptr(),
+            w.numel(), float(eps), group, int(gate_first), float(out_scale), out.data_ptr(), out.stride(0), _is16(out),
+            T, C, N.stream_ptr())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ feed-forward
+def glu(a: torch.Tensor, b: torch.Tensor, bias_a: torch.Tensor | None, bias_b: torch.Tensor | None, out: torch.Tensor,
+        scale: torch.Tensor | None = None, group: int = 0, scale_sigmoid: bool = False):
+    """out = silu(a + bias_a) * (b + bias_b) [* factor]; a, b fp32 [T, F] column slices, out fp32 or bf16 [T, F] (may
+    be a column slice). `scale` fp32 [T, F / group] (column slice allowed) gives one factor per row and group of
+    `group` columns, passed through a sigmoid first with `scale_sigmoid`."""
+    T, Fn = a.shape
+    if T == 0 or Fn == 0:
+        return out
+    if not a.is_cuda:
+        x = a.float() + bias_a if bias_a is not None else a.float()
+        y = b.float() + bias_b if bias_b is not None else b.float()
+        z = F.silu(x) * y
+        if scale is not None:
+            s = torch.sigmoid(scale.float()) if scale_sigmoid else scale.float()
+            z = (z.reshape(T, Fn // group, group) * s[:, :, None]).reshape(T, Fn)
+        out.copy_(z.to(out.dtype))
+        return out
+    _f32c(a, "glu")
+    _f32c(b, "glu")
+    if scale is not None and (group <= 0 or Fn % group or scale.shape[1] != Fn // group):
+        raise ValueError("glu: one factor per row and group of columns")
+    N.kcall("mxh_glu", a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), N.ptr(bias_a), N.ptr(bias_b),
+            N.ptr(scale), scale.stride(0) if scale is not None else 0, group if scale is not None else Fn,
+            int(scale_sigmoid), out.data_ptr(), out.stride(0), _is16(out), T, Fn, N.stream_ptr())
+    return out
+
+
+def moe_route(logits: torch.Tensor, top: int, scale: float, weights: torch.Tensor, eps: float = 1e-20):
+    """Router of a mixture of experts: s = softmax(logits) over all E experts, the `top` largest are kept, divided by
+    their sum (+ eps) and multiplied by `scale`. logits fp32 [T, E] (column slice allowed); weights fp32 [T, E]
+    contiguous: the chosen experts' weights, 0 elsewhere. Ties go to the lower expert index."""
+    T, E = logits.shape
+    if T == 0:
+        return weights
+    if not 0 < top <= E:
+        raise ValueError("moe_route: 1 <= top <= experts")
+    if not logits.is_cuda:
+        s = torch.softmax(logits.float(), -1)
+        tv, ti = torch.topk(s, top, dim=-1)
+        weights.zero_()
+        weights.scatter_(1, ti, tv / (tv.sum(-1, keepdim=True) + eps) * scale)
+        return weights
+    _f32c(logits, "moe_route")
+    if E > 1024:
+        raise ValueError("moe_route: at most 1024 experts")
+    N.kcall("mxh_moe_route", logits.data_ptr(), logits.stride(0), T, E, top, float(scale), float(eps),
+            weights.data_ptr(), N.stream_ptr())
+    return weights
