@@ -1,0 +1,474 @@
+// hybrid_ops.hip: the fp32 row kernels of hybrid attention / recurrent decoders (ops/hybrid.py): embedding gather,
+// offset RMS norm, rotary + head norm + paged append, causal convolution with carried tails, unit-length heads,
+// decay / write-strength coefficients, gated group norm, gated linear unit with per-group factors, expert routing.
+//
+// All statistics, angles, gates, routing and the residual are fp32; 16-bit (bf16) appears only on outputs that feed a
+// GEMM and in the paged pools. Launchers are `extern "C" int mxh_*(..., hipStream_t)`, return the launch's
+// hipError_t, never allocate or synchronise (safe under stream capture) and check the shapes their grids assume.
+#include "../mx_common.h"
+
+namespace {
+
+constexpr int NT = 256;
+
+template <bool B16>
+MX_DEV float ld_elem(const void* p, long i) {
+    if constexpr (B16) return bf16_to_f32(((const bf16_t*)p)[i]);
+    else return ((const float*)p)[i];
+}
+template <bool B16>
+MX_DEV void st_elem(void* p, long i, float v) {
+    if constexpr (B16) ((bf16_t*)p)[i] = f32_to_bf16(v);
+    else ((float*)p)[i] = v;
+}
+
+MX_DEV float silu_acc(float x) { return x / (1.f + expf(-x)); }
+MX_DEV float sigmoid_acc(float x) { return 1.f / (1.f + expf(-x)); }
+MX_DEV float softplus_acc(float x) { return x > 30.f ? x : log1pf(expf(x)); }
+
+// sum over the threads of a block of blockDim.x = 64 * k threads (k <= 4), returned to every thread
+MX_DEV float block_sum_dyn(float v, float* red) {
+    v = wave_sum(v);
+    const int nw = blockDim.x >> 6;
+    if (nw == 1) return v;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float s = 0.f;
+    for (int i = 0; i < nw; ++i) s += red[i];
+    return s;
+}
+
+template <bool B16>
+__global__ __launch_bounds__(NT) void embed_rows_kernel(const void* table, int V, const int* tokens, float* out,
+                                                        int ldo, int accumulate, int C) {
+    const int t = blockIdx.x;
+    int tok = tokens[t];
+    if (tok < 0 || tok >= V) tok = 0;
+    const long base = (long)tok * C;
+    float* o = out + (long)t * ldo;
+    for (int c = threadIdx.x; c < C; c += NT) {
+        const float v = ld_elem<B16>(table, base + c);
+        o[c] = accumulate ? o[c] + v : v;
+    }
+}
+
+constexpr int RC = 16;  // rows of up to NT * RC numbers are read once and kept in registers
+
+__global__ __launch_bounds__(NT) void offset_norm_kernel(const float* x, int ldx, const int* rows, const float* w,
+                                                         float offset, float eps, float* o32, int ld32, bf16_t* o16,
+                                                         int ld16, int C) {
+    __shared__ float red[NT / 64];
+    const int i = blockIdx.x;
+    const float* xr = x + (long)(rows ? rows[i] : i) * ldx;
+    const bool cached = C <= NT * RC;
+    float keep[RC];
+    float ss = 0.f;
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {  // clamped addresses: straight-line loads, all in flight together
+            const int c = threadIdx.x + k * NT;
+            const float v = xr[min(c, C - 1)];
+            keep[k] = c < C ? v : 0.f;
+            ss += keep[k] * keep[k];
+        }
+    } else {
+        for (int c = threadIdx.x; c < C; c += NT) {
+            const float v = xr[c];
+            ss += v * v;
+        }
+    }
+    ss = block_sum_dyn(ss, red);
+    const float sc = 1.f / sqrtf(ss / (float)C + eps);
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {
+            const int c = threadIdx.x + k * NT;
+            if (c < C) {
+                const float v = keep[k] * sc * (offset + w[c]);
+                if (o32) o32[(long)i * ld32 + c] = v;
+                if (o16) o16[(long)i * ld16 + c] = f32_to_bf16(v);
+            }
+        }
+        return;
+    }
+    for (int c = threadIdx.x; c < C; c += NT) {
+        const float v = xr[c] * sc * (offset + w[c]);
+        if (o32) o32[(long)i * ld32 + c] = v;
+        if (o16) o16[(long)i * ld16 + c] = f32_to_bf16(v);
+    }
+}
+
+// grid (T, H + 2G), one wave per (token, head): query heads, then key heads, then value heads. Element e < rot_dims
+// of a query / key head turns with its neighbour e ^ 1 by angle pos * base^(-(e / 2) * 2 / rot_dims).
+constexpr int HEAD_E = 8;  // elements per lane: heads of up to 512 numbers
+template <bool Q16, bool C16>
+__global__ __launch_bounds__(64) void rope_norm_append_kernel(const float* qi, const float* ki, const float* vi,
+                                                              int ldq, int ldk, int ldv, const int* positions, int H,
+                                                              int G, int dk, int dv, int rot, float neg_log_base,
+                                                              int norm, float eps, void* qo, int ldqo, void* kc,
+                                                              void* vc, const int* slots) {
+    const int t = blockIdx.x, u = blockIdx.y, lane = threadIdx.x;
+    if (u >= H + G) {  // value head: plain copy into the pool
+        const int sl = slots[t];
+        if (sl < 0) return;
+        const int g = u - H - G;
+        const float* src = vi + (long)t * ldv + (long)g * dv;
+        const long dst = ((long)sl * G + g) * dv;
+        for (int e = lane; e < dv; e += 64) st_elem<C16>(vc, dst + e, src[e]);
+        return;
+    }
+    const bool isq = u < H;
+    const int hd = isq ? u : u - H;
+    int sl = 0;
+    if (!isq) {
+        sl = slots[t];
+        if (sl < 0) return;
+    }
+    const float* src = isq ? qi + (long)t * ldq + (long)hd * dk : ki + (long)t * ldk + (long)hd * dk;
+    const float pos = (float)positions[t];
+    float val[HEAD_E];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < HEAD_E; ++k) {
+        const int e = lane + k * 64;
+        float v = 0.f;
+        if (e < dk) {
+            v = src[e];
+            if (e < rot) {
+                const float other = src[e ^ 1];
+                const float f = expf((float)(e >> 1) * (2.f / (float)rot) * neg_log_base);
+                float s, c;
+                sincosf(pos * f, &s, &c);
+                v = (e & 1) ? v * c + other * s : v * c - other * s;
+            }
+        }
+        val[k] = v;
+        ss += v * v;
+    }
+    float sc = 1.f;
+    if (norm) sc = 1.f / sqrtf(wave_sum(ss) / (float)dk + eps);
+    const long dst = isq ? (long)t * ldqo + (long)hd * dk : ((long)sl * G + hd) * dk;
+#pragma unroll
+    for (int k = 0; k < HEAD_E; ++k) {
+        const int e = lane + k * 64;
+        if (e < dk) {
+            if (isq) st_elem<Q16>(qo, dst + e, val[k] * sc);
+            else st_elem<C16>(kc, dst + e, val[k] * sc);
+        }
+    }
+}
+
+// grid (ceil(C / NT), sequences, ceil(T / CONV_ROWS)): thread = channel. Reads the tails only; conv_tails_kernel
+// rolls them afterwards
+constexpr int CONV_ROWS = 32;
+__global__ __launch_bounds__(NT) void causal_conv_kernel(const float* x, int ldx, const float* w, const float* bias,
+                                                         int taps, int silu, float* tails, const int* state,
+                                                         const int* positions, int n_dec, const int* pf_cu, float* out,
+                                                         int ldo, int C) {
+    const int c = blockIdx.x * NT + threadIdx.x;
+    const int s = blockIdx.y;
+    int row0, n;
+    if (s < n_dec) {
+        row0 = s;
+        n = 1;
+    } else {
+        const int k = s - n_dec;
+        row0 = n_dec + pf_cu[k];
+        n = pf_cu[k + 1] - pf_cu[k];
+    }
+    const int t0 = blockIdx.z * CONV_ROWS;
+    if (t0 >= n || c >= C) return;
+    const int slot = state[s];
+    const int nt = taps - 1;
+    const bool fresh = positions[row0] == 0 || slot < 0;
+    float* tail = tails + ((long)(slot < 0 ? 0 : slot) * (nt > 0 ? nt : 1)) * C + c;  // entry i at tail[i * C]
+    float wr[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) wr[j] = j < taps ? w[(long)c * taps + j] : 0.f;
+    const float b = bias ? bias[c] : 0.f;
+    const int t1 = min(n, t0 + CONV_ROWS);
+    for (int t = t0; t < t1; ++t) {
+        float acc = b;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            if (j < taps) {
+                const int tau = t - nt + j;  // input index within the chunk; < 0: carried from earlier steps
+                float v;
+                if (tau >= 0) v = x[(long)(row0 + tau) * ldx + c];
+                else v = fresh ? 0.f : tail[(long)(nt + tau) * C];
+                acc += wr[j] * v;
+            }
+        }
+        out[(long)(row0 + t) * ldo + c] = silu ? silu_acc(acc) : acc;
+    }
+}
+
+// second pass of the convolution (launched after it on the same stream): new tails = last taps-1 inputs
+__global__ __launch_bounds__(NT) void conv_tails_kernel(const float* x, int ldx, int taps, float* tails, const int* state,
+                                                        const int* positions, int n_dec, const int* pf_cu, int C) {
+    const int c = blockIdx.x * NT + threadIdx.x;
+    const int s = blockIdx.y;
+    int row0, n;
+    if (s < n_dec) {
+        row0 = s;
+        n = 1;
+    } else {
+        const int k = s - n_dec;
+        row0 = n_dec + pf_cu[k];
+        n = pf_cu[k + 1] - pf_cu[k];
+    }
+    const int slot = state[s];
+    const int nt = taps - 1;
+    if (c >= C || n <= 0 || slot < 0 || nt <= 0) return;
+    const bool fresh = positions[row0] == 0;
+    float* tail = tails + (long)slot * nt * C + c;
+    for (int i = 0; i < nt; ++i) {
+        const int tau = n - nt + i;
+        float v;
+        if (tau >= 0) v = x[(long)(row0 + tau) * ldx + c];
+        else v = fresh ? 0.f : tail[(long)(nt + tau) * C];  // index n + i > i: not yet overwritten
+        tail[(long)i * C] = v;
+    }
+}
+
+// grid (T, heads), one wave per head
+__global__ __launch_bounds__(64) void unit_norm_kernel(float* x, int ldx, int dim, float eps, float scale) {
+    float* p = x + (long)blockIdx.x * ldx + (long)blockIdx.y * dim;
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < dim; e += 64) ss += p[e] * p[e];
+    const float sc = scale / sqrtf(wave_sum(ss) + eps);
+    for (int e = threadIdx.x; e < dim; e += 64) p[e] *= sc;
+}
+
+__global__ __launch_bounds__(NT) void scan_coefs_kernel(const float* a, int lda, const float* b, int ldb,
+                                                        const float* A_log, const float* dt_bias, float* decay,
+                                                        float* coef, int T, int H) {
+    const int i = blockIdx.x * NT + threadIdx.x;
+    if (i >= T * H) return;
+    const int t = i / H, h = i - t * H;
+    const float s = softplus_acc(a[(long)t * lda + h] + dt_bias[h]);
+    decay[i] = expf(-expf(A_log[h]) * s);
+    coef[i] = b ? sigmoid_acc(b[(long)t * ldb + h]) : s;
+}
+
+// grid (T, C / group): one block per (token, group of columns)
+template <bool B16>
+__global__ void gated_group_norm_kernel(const float* y, int ldy, const float* gate, int ldg, const float* w, int wlen,
+                                        float eps, int group, int gate_first, float out_scale, void* out, int ldo) {
+    __shared__ float red[NT / 64];
+    const int t = blockIdx.x, c0 = blockIdx.y * group;
+    const float* yr = y + (long)t * ldy + c0;
+    const float* gr = gate + (long)t * ldg + c0;
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < group; e += blockDim.x) {
+        float v = yr[e];
+        if (gate_first) v *= silu_acc(gr[e]);
+        ss += v * v;
+    }
+    ss = block_sum_dyn(ss, red);
+    const float sc = out_scale / sqrtf(ss / (float)group + eps);
+    for (int e = threadIdx.x; e < group; e += blockDim.x) {
+        const float g = silu_acc(gr[e]);
+        float v = yr[e];
+        if (gate_first) v *= g;
+        v = v * sc * w[(c0 + e) % wlen];
+        if (!gate_first) v *= g;
+        st_elem<B16>(out, (long)t * ldo + c0 + e, v);
+    }
+}
+
+// grid (T, ceil(F / NT))
+template <bool B16>
+__global__ __launch_bounds__(NT) void glu_kernel(const float* a, int lda, const float* b, int ldb, const float* ba,
+                                                 const float* bb, const float* scale, int lds, int group,
+                                                 int scale_sigmoid, void* out, int ldo, int F) {
+    const int f = blockIdx.y * NT + threadIdx.x, t = blockIdx.x;
+    if (f >= F) return;
+    float fac = 1.f;
+    if (scale) {
+        fac = scale[(long)t * lds + f / group];
+        if (scale_sigmoid) fac = sigmoid_acc(fac);
+        if (fac == 0.f) {  // an expert the router did not choose: nothing to evaluate
+            st_elem<B16>(out, (long)t * ldo + f, 0.f);
+            return;
+        }
+    }
+    const float x = a[(long)t * lda + f] + (ba ? ba[f] : 0.f);
+    const float y = b[(long)t * ldb + f] + (bb ? bb[f] : 0.f);
+    st_elem<B16>(out, (long)t * ldo + f, silu_acc(x) * y * fac);
+}
+
+// one wave per token; lane l holds experts l, l + 64, ... (up to 16 each)
+constexpr int ROUTE_E = 16;
+__global__ __launch_bounds__(64) void moe_route_kernel(const float* logits, int ld, int E, int top, float scale,
+                                                       float eps, float* weights) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* z = logits + (long)t * ld;
+    float v[ROUTE_E];
+    float m = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < ROUTE_E; ++k) {
+        const int e = lane + k * 64;
+        v[k] = e < E ? z[e] : -INFINITY;
+        m = fmaxf(m, v[k]);
+    }
+    m = wave_max(m);
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < ROUTE_E; ++k) {
+        v[k] = (lane + k * 64) < E ? expf(v[k] - m) : -1.f;  // scores are >= 0; -1 marks absent or taken
+        sum += fmaxf(v[k], 0.f);
+    }
+    sum = wave_sum(sum);
+    float* wr = weights + (long)t * E;
+    for (int e = lane; e < E; e += 64) wr[e] = 0.f;
+    float mine[ROUTE_E];  // score of the experts this lane holds that were chosen (else 0)
+#pragma unroll
+    for (int k = 0; k < ROUTE_E; ++k) mine[k] = 0.f;
+    float chosen = 0.f;
+    for (int r = 0; r < top; ++r) {
+        float best = -1.f;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int k = 0; k < ROUTE_E; ++k) {
+            if (v[k] > best) {  // strict: the lowest index of equal scores within the lane
+                best = v[k];
+                bi = lane + k * 64;
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (ob > best || (ob == best && oi < bi)) {
+                best = ob;
+                bi = oi;
+            }
+        }
+        chosen += best / sum;
+#pragma unroll
+        for (int k = 0; k < ROUTE_E; ++k) {
+            if (lane + k * 64 == bi) {
+                mine[k] = v[k] / sum;
+                v[k] = -1.f;
+            }
+        }
+    }
+    const float norm = scale / (chosen + eps);
+#pragma unroll
+    for (int k = 0; k < ROUTE_E; ++k) {
+        const int e = lane + k * 64;
+        if (e < E && v[k] < 0.f) wr[e] = mine[k] * norm;  // the taken ones (absent ones have e >= E)
+    }
+}
+
+}  // namespace
+
+#define MXH_CHECK(cond) \
+    if (!(cond)) return (int)hipErrorInvalidValue
+
+extern "C" int mxh_embed_rows(const void* table, int is16, int V, const int* tokens, float* out, int ldo,
+                              int accumulate, int T, int C, hipStream_t st) {
+    if (T <= 0) return 0;
+    MXH_CHECK(table && tokens && out && C > 0 && V > 0 && ldo >= C);
+    if (is16) embed_rows_kernel<true><<<T, NT, 0, st>>>(table, V, tokens, out, ldo, accumulate, C);
+    else embed_rows_kernel<false><<<T, NT, 0, st>>>(table, V, tokens, out, ldo, accumulate, C);
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_offset_norm(const float* x, int ldx, const int* rows, const float* w, float offset, float eps,
+                               float* o32, int ld32, bf16_t* o16, int ld16, int M, int C, hipStream_t st) {
+    if (M <= 0) return 0;
+    MXH_CHECK(x && w && (o32 || o16) && C > 0 && ldx >= C && (!o32 || ld32 >= C) && (!o16 || ld16 >= C));
+    offset_norm_kernel<<<M, NT, 0, st>>>(x, ldx, rows, w, offset, eps, o32, ld32, o16, ld16, C);
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_rope_norm_append(const float* qi, const float* ki, const float* vi, int ldq, int ldk, int ldv,
+                                    const int* positions, int H, int G, int dk, int dv, int rot, float base, int norm,
+                                    float eps, void* qo, int ldqo, int q16, void* kc, void* vc, int c16,
+                                    const int* slots, int T, hipStream_t st) {
+    if (T <= 0) return 0;
+    MXH_CHECK(qi && ki && vi && positions && qo && kc && vc && slots);
+    MXH_CHECK(H > 0 && G > 0 && dk > 0 && dv > 0 && dk <= 64 * HEAD_E && rot >= 0 && rot <= dk && rot % 2 == 0);
+    MXH_CHECK(ldq >= H * dk && ldk >= G * dk && ldv >= G * dv && ldqo >= H * dk && base > 0.f);
+    const dim3 grid(T, H + 2 * G);
+    const float nlb = -logf(base);
+#define GO(Q, C)                                                                                                   \
+    rope_norm_append_kernel<Q, C><<<grid, 64, 0, st>>>(qi, ki, vi, ldq, ldk, ldv, positions, H, G, dk, dv, rot, nlb, \
+                                                       norm, eps, qo, ldqo, kc, vc, slots)
+    if (q16 && c16) GO(true, true);
+    else if (q16) GO(true, false);
+    else if (c16) GO(false, true);
+    else GO(false, false);
+#undef GO
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_causal_conv(const float* x, int ldx, const float* w, const float* bias, int taps, int silu,
+                               float* tails, const int* state, const int* positions, int n_dec, const int* pf_cu,
+                               int n_pf, float* out, int ldo, int T, int C, hipStream_t st) {
+    if (T <= 0) return 0;
+    MXH_CHECK(x && w && tails && state && positions && out && C > 0 && taps >= 1 && taps <= 16);
+    MXH_CHECK(ldx >= C && ldo >= C && n_dec >= 0 && n_pf >= 0 && n_dec + n_pf > 0 && (n_pf == 0 || pf_cu));
+    const int rows = n_pf ? T - n_dec : 1;
+    const dim3 grid((C + NT - 1) / NT, n_dec + n_pf, (max(rows, 1) + CONV_ROWS - 1) / CONV_ROWS);
+    causal_conv_kernel<<<grid, NT, 0, st>>>(x, ldx, w, bias, taps, silu, tails, state, positions, n_dec, pf_cu, out,
+                                            ldo, C);
+    if (taps > 1) {
+        const dim3 g2((C + NT - 1) / NT, n_dec + n_pf);
+        conv_tails_kernel<<<g2, NT, 0, st>>>(x, ldx, taps, tails, state, positions, n_dec, pf_cu, C);
+    }
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_unit_norm(float* x, int ldx, int heads, int dim, float eps, float scale, int T, hipStream_t st) {
+    if (T <= 0) return 0;
+    MXH_CHECK(x && heads > 0 && dim > 0 && ldx >= heads * dim);
+    unit_norm_kernel<<<dim3(T, heads), 64, 0, st>>>(x, ldx, dim, eps, scale);
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_scan_coefs(const float* a, int lda, const float* b, int ldb, const float* A_log,
+                              const float* dt_bias, float* decay, float* coef, int T, int H, hipStream_t st) {
+    if (T <= 0) return 0;
+    MXH_CHECK(a && A_log && dt_bias && decay && coef && H > 0 && lda >= H && (!b || ldb >= H));
+    scan_coefs_kernel<<<(T * H + NT - 1) / NT, NT, 0, st>>>(a, lda, b, ldb, A_log, dt_bias, decay, coef, T, H);
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_gated_group_norm(const float* y, int ldy, const float* gate, int ldg, const float* w, int wlen,
+                                    float eps, int group, int gate_first, float out_scale, void* out, int ldo,
+                                    int o16, int T, int C, hipStream_t st) {
+    if (T <= 0) return 0;
+    MXH_CHECK(y && gate && w && out && C > 0 && group > 0 && C % group == 0 && wlen > 0 && C % wlen == 0);
+    MXH_CHECK(ldy >= C && ldg >= C && ldo >= C);
+    const dim3 grid(T, C / group);
+    const int nt = group <= 256 ? 64 : NT;
+    if (o16) gated_group_norm_kernel<true><<<grid, nt, 0, st>>>(y, ldy, gate, ldg, w, wlen, eps, group, gate_first,
+                                                                out_scale, out, ldo);
+    else gated_group_norm_kernel<false><<<grid, nt, 0, st>>>(y, ldy, gate, ldg, w, wlen, eps, group, gate_first,
+                                                             out_scale, out, ldo);
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_glu(const float* a, int lda, const float* b, int ldb, const float* ba, const float* bb,
+                       const float* scale, int lds, int group, int scale_sigmoid, void* out, int ldo, int o16, int T,
+                       int F, hipStream_t st) {
+    if (T <= 0 || F <= 0) return 0;
+    MXH_CHECK(a && b && out && lda >= F && ldb >= F && ldo >= F && group > 0 && F <= 65535 * NT);
+    MXH_CHECK(!scale || (F % group == 0 && lds >= F / group));
+    const dim3 grid(T, (F + NT - 1) / NT);
+    if (o16) glu_kernel<true><<<grid, NT, 0, st>>>(a, lda, b, ldb, ba, bb, scale, lds, group, scale_sigmoid, out, ldo, F);
+    else glu_kernel<false><<<grid, NT, 0, st>>>(a, lda, b, ldb, ba, bb, scale, lds, group, scale_sigmoid, out, ldo, F);
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_moe_route(const float* logits, int ld, int T, int E, int top, float scale, float eps,
+                             float* weights, hipStream_t st) {
+    if (T <= 0) return 0;
+    MXH_CHECK(logits && weights && E > 0 && E <= 64 * ROUTE_E && top > 0 && top <= E && ld >= E);
+    moe_route_kernel<<<T, 64, 0, st>>>(logits, ld, E, top, scale, eps, weights);
+    return (int)hipGetLastError();
+}

@@ -156,6 +156,18 @@ def build_latent(verbose=False) -> Path:
     return _build_lib("libmxl.so", srcs, headers, HIPCC, cflags, ["-fPIC"], verbose)
 
 
+def build_hybrid(verbose=False) -> Path:
+    """libmxh.so: the kernels of the hybrid attention / recurrent decoders (csrc/kernels/hybrid/), a library of its
+    own for the same reason as libmxl.so."""
+    kdir = CSRC / "kernels"
+    srcs = sorted((kdir / "hybrid").glob("*.hip"))
+    headers = sorted(kdir.glob("*.h"))
+    cflags = [f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17", "-ffp-contract=fast",
+              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-I", str(kdir), "-Wno-unused-result",
+              "-Wno-unknown-warning-option"]
+    return _build_lib("libmxh.so", srcs, headers, HIPCC, cflags, ["-fPIC"], verbose)
+
+
 def build_runtime(verbose=False) -> Path:
     rdir = CSRC / "runtime"
     srcs = sorted(rdir.glob("*.cpp"))
@@ -175,6 +187,7 @@ def build_all(verbose=False):
         raise RuntimeError(f"hipcc not found at {HIPCC}")
     k = build_kernels(verbose)
     build_latent(verbose)
+    build_hybrid(verbose)
     r = build_runtime(verbose)
     return k, r
 

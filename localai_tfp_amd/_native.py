@@ -140,6 +140,35 @@ LATENT_SIGS = {
     "mxl_head_gate_pack": [P, P, I, P, I, I, I, I, I, P],
 }
 
+# libmxh.so (csrc/kernels/hybrid/): kernels of the hybrid attention / recurrent decoders (ops/hybrid.py)
+HYBRID_SIGS = {
+    # table, is16, V, tokens, out, ldo, accumulate, T, C, stream
+    "mxh_embed_rows": [P, I, I, P, P, I, I, I, I, P],
+    # x, ldx, rows, w, offset, eps, out32, ld32, out16, ld16, M, C, stream
+    "mxh_offset_norm": [P, I, P, P, F, F, P, I, P, I, I, I, P],
+    # q, k, v, ldq, ldk, ldv, positions, H, G, dk, dv, rot_dims, base, norm, eps, q_out, ldqo, q16, kc, vc, c16, slots,
+    # T, stream
+    "mxh_rope_norm_append": [P, P, P, I, I, I, P, I, I, I, I, I, F, I, F, P, I, I, P, P, I, P, I, P],
+    # q, ldq, q16, kc, vc, bs, bt, bt_stride, cu_q, ctx, n_seqs, n_rows, row_base, out, ldo, o16, H, G, dk, dv, scale,
+    # chunk, window, sink, out_scale, stream
+    "mxh_attention": [P, I, I, P, P, I, P, I, P, P, I, I, I, P, I, I, I, I, I, I, F, I, I, I, F, P],
+    # x, ldx, w, bias, taps, silu, tails, state, positions, n_dec, pf_cu, n_pf, out, ldo, T, C, stream
+    "mxh_causal_conv": [P, I, P, P, I, I, P, P, P, I, P, I, P, I, I, I, P],
+    # x, ldx, heads, dim, eps, scale, T, stream
+    "mxh_unit_norm": [P, I, I, I, F, F, I, P],
+    # a, lda, b, ldb, A_log, dt_bias, decay, coef, T, H, stream
+    "mxh_scan_coefs": [P, I, P, I, P, P, P, P, I, I, P],
+    # k, ldk, q, ldq, v, ldv, decay, coef, skip, state, seq_state, positions, n_dec, pf_cu, n_pf, out, ldo, H, G, N, P,
+    # delta, stream
+    "mxh_state_scan": [P, I, P, I, P, I, P, P, P, P, P, P, I, P, I, P, I, I, I, I, I, I, P],
+    # y, ldy, gate, ldg, w, wlen, eps, group, gate_first, out_scale, out, ldo, o16, T, C, stream
+    "mxh_gated_group_norm": [P, I, P, I, P, I, F, I, I, F, P, I, I, I, I, P],
+    # a, lda, b, ldb, bias_a, bias_b, scale, lds, group, scale_sigmoid, out, ldo, o16, T, F, stream
+    "mxh_glu": [P, I, P, I, P, P, P, I, I, I, P, I, I, I, I, P],
+    # logits, ld, T, E, top, scale, eps, weights, stream
+    "mxh_moe_route": [P, I, I, I, I, F, F, P, P],
+}
+
 HIP_ERRORS = {1: "hipErrorInvalidValue", 2: "hipErrorOutOfMemory", 98: "hipErrorInvalidDeviceFunction",
               209: "hipErrorNoBinaryForGpu", 700: "hipErrorIllegalAddress", 719: "hipErrorLaunchFailure"}
 
@@ -200,14 +229,34 @@ def latent_kernels():
     return _latent
 
 
+_hybrid = None
+
+
+def hybrid_kernels():
+    """Load libmxh.so (hybrid attention / recurrent decoder kernels), building it first when the tree has none.
+    Raises NativeError if it cannot be built or loaded."""
+    global _hybrid
+    if _hybrid is None:
+        with _lock:
+            if _hybrid is None:
+                ensure_built("hybrid")
+                lib = _load("libmxh.so")
+                for n, sig in HYBRID_SIGS.items():
+                    fn = getattr(lib, n)
+                    fn.argtypes = sig
+                    fn.restype = C.c_int
+                _hybrid = lib
+    return _hybrid
+
+
 def ensure_built(group: str) -> None:
     """Build a native library of the tree if it is not there yet (never rebuilds one that is)."""
-    name = {"latent": "libmxl.so"}[group]
+    name = {"latent": "libmxl.so", "hybrid": "libmxh.so"}[group]
     if (_LIBDIR / name).exists():
         return
     from . import _build
     try:
-        {"latent": _build.build_latent}[group]()
+        {"latent": _build.build_latent, "hybrid": _build.build_hybrid}[group]()
     except Exception as ex:
         raise NativeError(f"could not build {name}: {ex}") from ex
 
@@ -248,7 +297,7 @@ def ensure_act(dtype) -> None:
 
 
 def kcall(name: str, *args):
-    lib = latent_kernels() if name.startswith("mxl_") else kernels()
+    lib = latent_kernels() if name.startswith("mxl_") else hybrid_kernels() if name.startswith("mxh_") else kernels()
     fn = getattr(lib, name, None)
     if fn is None:
         raise NativeError(f"{name} not exported by {lib._name} (stale build?)")
@@ -273,7 +322,7 @@ def ptr(t) -> int | None:
 def loaded_library_paths():
     """Paths of the native libraries loaded into this process (for diagnostics / tests)."""
     out = []
-    for lib in (_kernels, _runtime, _latent):
+    for lib in (_kernels, _runtime, _latent, _hybrid):
         if lib is not None:
             out.append(lib._name)
     return out

@@ -33,13 +33,11 @@ def main(argv=None) -> int:
 
     import numpy as np
     import torch
-    from .. import _native
     from ..engine.engine import EngineConfig, LLMEngine
     from ..models.loader import load_llm
 
     dev = a.device or ("cuda" if torch.cuda.is_available() else "cpu")
-    if dev.startswith("cuda"):
-        _native.ensure_built("latent")
+    if dev.startswith("cuda"):  # the model's kernel library is built at its first launch if the tree has none
         torch.backends.cuda.matmul.allow_tf32 = False
     dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[a.dtype]
     model, tok, _cfg, _ = load_llm(a.model, torch.device(dev), overrides={"dtype": dtype})
