@@ -96,13 +96,14 @@ def parse():
                     help="comma list of sampling phases measured back to back on the same server: reference = "
                          "the reference's defaults (temperature 0.9, top_k 40, top_p 0.95; backend_config.go "
                          "SetDefaults) on the GPU sampler; greedy = argmax. The first phase is the headline")
-    ap.add_argument("--arch-bench", default="", choices=["", "vosotar"],
+    ap.add_argument("--arch-bench", default="", choices=["", "vosotar", "vugotar"],
                     help="instead of the headline serving benchmark: prefill and decode throughput of this model "
                          "family beside the Llama graph at equal layer sizes (random bf16 / f16 weights, one GPU)")
     ap.add_argument("--arch-sizes", default="1b,7b", help="--arch-bench: comma list of layer sizes (1b, 7b)")
     ap.add_argument("--arch-layers", type=int, default=4, help="--arch-bench: layers per model")
-    ap.add_argument("--arch-models", default="", help="--arch-bench: comma list to restrict the models (vosotar, llama-f16)")
+    ap.add_argument("--arch-models", default="", help="--arch-bench: comma list to restrict the models (vosotar, vugotar, llama-f16)")
     ap.add_argument("--arch-batches", default="1,32", help="--arch-bench: decode batch sizes")
+    ap.add_argument("--arch-chunk", type=int, default=2048, help="--arch-bench vugotar: attention chunk size")
     return ap.parse_args()
 
 
@@ -233,9 +234,22 @@ def run_arch_bench(args) -> int:
 
     def models(sz):
         s = ARCH_SIZES[sz]
-        vc = VO.make_config(hidden=s["hidden"], vocab=V, n_layers=nl, heads=s["heads"], dim=128, vdim=128, kv_rank=512,
-                            q_rank=s["q_rank"], ff=s["ff"], name=f"vosotar-{sz}")
-        yield "vosotar", lambda: VO.VosotarModel.load(vc, VO.synthetic_source(vc, 1), dev, torch.bfloat16)
+        if args.arch_bench == "vugotar":
+            # attention + delta-rule layers with a state-space layer every fourth, dense feed-forwards; attention
+            # heads as the Llama graph's (GQA 4:1, head size 128), delta rule with half as many heads of 128 x 128
+            # states, state-space layer twice as wide as the model with 128 states per head
+            from localai_tfp_amd.models import vugotar as VU
+            pat = tuple("mamba2" if i % 4 == 3 else "parallel" for i in range(nl))
+            uc = VU.make_config(hidden=s["hidden"], vocab=V, pattern=pat, mlps=("dense",), heads=s["heads"],
+                                kv_heads=max(1, s["heads"] // 4), dim=128, vdim=128, chunk=args.arch_chunk,
+                                d_heads=s["heads"] // 2, d_kv_heads=max(1, s["heads"] // 4), d_dim=128, d_vdim=128,
+                                d_conv=4, m_heads=2 * s["hidden"] // 64, m_vdim=64, m_state=128, m_groups=1,
+                                m_norm_groups=1, m_conv=4, ff=s["ff"], name=f"vugotar-{sz}")
+            yield "vugotar", lambda: VU.VugotarModel.load(uc, VU.synthetic_source(uc, 1), dev, torch.bfloat16)
+        else:
+            vc = VO.make_config(hidden=s["hidden"], vocab=V, n_layers=nl, heads=s["heads"], dim=128, vdim=128,
+                                kv_rank=512, q_rank=s["q_rank"], ff=s["ff"], name=f"vosotar-{sz}")
+            yield "vosotar", lambda: VO.VosotarModel.load(vc, VO.synthetic_source(vc, 1), dev, torch.bfloat16)
         lc = LlamaConfig(name=f"llama-{sz}", n_layers=nl, hidden=s["hidden"], ffn=s["ff"], n_heads=s["heads"],
                          n_kv_heads=max(1, s["heads"] // 4), head_dim=128, vocab=V, ctx_train=8192, rope_base=10000.0,
                          rope_dim=128)
