@@ -7,6 +7,12 @@
 // running maximum and sum (fp32), and the lanes then share out the value columns, each accumulating
 // sum_j p_j v_j[c] for its columns over the tile's keys. Scores, softmax and accumulators are fp32 for both pool
 // formats. The sink is a virtual key of score 0 and value 0: the running maximum starts at 0 and the sum at 1.
+// With parts > 1 (decode rows of long contexts) grid.z splits a row's visible keys into partitions whose
+// (max, sum, unnormalised output) go to a workspace; attn_merge_kernel combines them in a fixed order and adds the sink.
+//
+// Long prompt chunks take another route (ops/hybrid.py): kv_gather_kernel copies the chunk's visible keys and values
+// from the pages into head-major matrices, head_transpose_kernel does the same for the queries, the library computes
+// the score and value products, and masked_softmax_kernel turns raw scores into masked, sink-normalised weights.
 #include "../mx_common.h"
 
 namespace {
@@ -55,12 +61,13 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
                                                        const int* bt, int bt_stride, const int* cu_q, const int* ctx,
                                                        int n_seqs, int row_base, void* out, int ldo, int H, int G,
                                                        int dk, int dv, float scale, int chunk, int window, int sink,
-                                                       float out_scale) {
+                                                       float out_scale, int row_off, int parts, int part_len,
+                                                       float* part_ml, float* part_o) {
     extern __shared__ float lds[];  // [dk] query, [64] weights, [64] row offsets (as int pairs)
     float* qs = lds;
     float* ps = lds + dk;
     long* rowoff = (long*)(ps + 64 + ((dk & 1) ? 1 : 0));
-    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int r = blockIdx.x + row_off, h = blockIdx.y, lane = threadIdx.x, z = blockIdx.z;
     int s, pos;
     if (!cu_q) {
         s = r;
@@ -79,7 +86,12 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
     const int g = h / (H / G);
     const long qrow = (long)(row_base + r) * ldq + (long)h * dk;
     for (int e = lane; e < dk; e += 64) qs[e] = ld1<B16>(q, qrow + e) * scale;
-    const int lo = chunk > 0 ? (pos / chunk) * chunk : window > 0 ? max(0, pos - window + 1) : 0;
+    int lo = chunk > 0 ? (pos / chunk) * chunk : window > 0 ? max(0, pos - window + 1) : 0;
+    if (parts > 1) {  // this partition's keys; the sink joins in the merge
+        lo += z * part_len;
+        pos = min(pos, lo + part_len - 1);
+        sink = 0;
+    }
     const int* table = bt + (long)s * bt_stride;
     float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
     float acc[DVU];
@@ -110,10 +122,31 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
             const int c = lane + u * 64;
             if (c < dv) {
                 float a = acc[u] * alpha;
-                for (int jj = 0; jj < nk; ++jj) a += ps[jj] * ld1<B16>(vc, rowoff[jj] + c);
+                int jj = 0;
+                for (; jj + 8 <= nk; jj += 8) {  // eight independent loads in flight, then their products
+                    float vv[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) vv[e] = ld1<B16>(vc, rowoff[jj + e] + c);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) a += ps[jj + e] * vv[e];
+                }
+                for (; jj < nk; ++jj) a += ps[jj] * ld1<B16>(vc, rowoff[jj] + c);
                 acc[u] = a;
             }
         }
+    }
+    if (parts > 1) {
+        const long pr = ((long)r * H + h) * parts + z;
+        if (lane == 0) {
+            part_ml[pr * 2] = m;
+            part_ml[pr * 2 + 1] = l;
+        }
+#pragma unroll
+        for (int u = 0; u < DVU; ++u) {
+            const int c = lane + u * 64;
+            if (c < dv) part_o[pr * dv + c] = acc[u];
+        }
+        return;
     }
     const float inv = out_scale / l;
     const long orow = (long)(row_base + r) * ldo + (long)h * dv;
@@ -127,6 +160,97 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
     }
 }
 
+// grid (rows, H): combines the partitions of a row in order; an empty partition has sum 0
+template <bool O16>
+__global__ __launch_bounds__(64) void attn_merge_kernel(const float* part_ml, const float* part_o, int parts, int H,
+                                                        int dv, int sink, float out_scale, int row_base, void* out,
+                                                        int ldo) {
+    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const long p0 = ((long)r * H + h) * parts;
+    float M = sink ? 0.f : -INFINITY;
+    for (int z = 0; z < parts; ++z)
+        if (part_ml[(p0 + z) * 2 + 1] > 0.f) M = fmaxf(M, part_ml[(p0 + z) * 2]);
+    float L = sink ? expf(-M) : 0.f;
+    float acc[DVU];
+#pragma unroll
+    for (int u = 0; u < DVU; ++u) acc[u] = 0.f;
+    for (int z = 0; z < parts; ++z) {
+        const float lz = part_ml[(p0 + z) * 2 + 1];
+        if (!(lz > 0.f)) continue;
+        const float w = expf(part_ml[(p0 + z) * 2] - M);
+        L += lz * w;
+#pragma unroll
+        for (int u = 0; u < DVU; ++u) {
+            const int c = lane + u * 64;
+            if (c < dv) acc[u] += part_o[(p0 + z) * dv + c] * w;
+        }
+    }
+    const float inv = out_scale / L;
+    const long orow = (long)(row_base + r) * ldo + (long)h * dv;
+#pragma unroll
+    for (int u = 0; u < DVU; ++u) {
+        const int c = lane + u * 64;
+        if (c < dv) {
+            if constexpr (O16) ((bf16_t*)out)[orow + c] = f32_to_bf16(acc[u] * inv);
+            else ((float*)out)[orow + c] = acc[u] * inv;
+        }
+    }
+}
+
+// grid (keys, G): key jj of the range is the token at position lo + jj of the sequence whose block table is `table`;
+// its group's key and value rows go to kh [G][n][dk] and vh [G][n][dv]
+template <typename E>
+__global__ __launch_bounds__(64) void kv_gather_kernel(const E* kc, const E* vc, int bs, const int* table, int lo, int n,
+                                                       int G, int dk, int dv, E* kh, E* vh) {
+    const int jj = blockIdx.x, g = blockIdx.y;
+    const int j = lo + jj;
+    const long tok = (long)table[j / bs] * bs + (j % bs);
+    const E* ks = kc + (tok * G + g) * dk;
+    const E* vs = vc + (tok * G + g) * dv;
+    E* kd = kh + ((long)g * n + jj) * dk;
+    E* vd = vh + ((long)g * n + jj) * dv;
+    for (int e = threadIdx.x; e < dk; e += 64) kd[e] = ks[e];
+    for (int e = threadIdx.x; e < dv; e += 64) vd[e] = vs[e];
+}
+
+// grid (n, H): dst[i * d_si + h * d_sh + e] = scale * src[i * s_si + h * s_sh + e], e < d
+template <bool S16, bool D16>
+__global__ __launch_bounds__(64) void head_transpose_kernel(const void* src, long s_si, long s_sh, void* dst, long d_si,
+                                                            long d_sh, int d, float scale) {
+    const long so = blockIdx.x * s_si + blockIdx.y * s_sh, dof = blockIdx.x * d_si + blockIdx.y * d_sh;
+    for (int e = threadIdx.x; e < d; e += 64) {
+        const float v = ld1<S16>(src, so + e) * scale;
+        if constexpr (D16) ((bf16_t*)dst)[dof + e] = f32_to_bf16(v);
+        else ((float*)dst)[dof + e] = v;
+    }
+}
+
+// grid (H * n): row (h, i) holds the raw scores of the query at position p0 + i against the keys at positions
+// key0 .. key0 + nk - 1. Writes the masked, sink-normalised softmax weights (zeros outside the visible range).
+template <bool P16>
+__global__ __launch_bounds__(256) void masked_softmax_kernel(const float* sc, void* pw, int n, int nk, int p0, int key0,
+                                                             float scale, int chunk, int window, int sink) {
+    __shared__ float red[4];
+    const long row = blockIdx.x;
+    const int i = (int)(row % n);
+    const int pos = p0 + i;
+    const int lo = chunk > 0 ? (pos / chunk) * chunk : window > 0 ? max(0, pos - window + 1) : 0;
+    const int a = max(lo, key0) - key0, b = min(pos - key0, nk - 1);  // visible local range [a, b]
+    const float* s = sc + row * nk;
+    float m = sink ? 0.f : -INFINITY;
+    for (int j = a + threadIdx.x; j <= b; j += 256) m = fmaxf(m, s[j] * scale);
+    m = block_max<256>(m, red);
+    float l = 0.f;
+    for (int j = a + threadIdx.x; j <= b; j += 256) l += expf(s[j] * scale - m);
+    l = block_sum<256>(l, red) + (sink ? expf(-m) : 0.f);
+    const float inv = 1.f / l;
+    for (int j = threadIdx.x; j < nk; j += 256) {
+        const float p = (j >= a && j <= b) ? expf(s[j] * scale - m) * inv : 0.f;
+        if constexpr (P16) ((bf16_t*)pw)[row * nk + j] = f32_to_bf16(p);
+        else ((float*)pw)[row * nk + j] = p;
+    }
+}
+
 }  // namespace
 
 #define MXH_CHECK(cond) \
@@ -135,21 +259,64 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
 extern "C" int mxh_attention(const void* q, int ldq, int q16, const void* kc, const void* vc, int bs, const int* bt,
                              int bt_stride, const int* cu_q, const int* ctx, int n_seqs, int n_rows, int row_base,
                              void* out, int ldo, int o16, int H, int G, int dk, int dv, float scale, int chunk,
-                             int window, int sink, float out_scale, hipStream_t st) {
+                             int window, int sink, float out_scale, int row_off, int parts, int part_len,
+                             float* part_ml, float* part_o, hipStream_t st) {
     if (n_rows <= 0 || n_seqs <= 0) return 0;
     MXH_CHECK(q && kc && vc && bt && ctx && out && bs > 0 && bt_stride > 0);
     MXH_CHECK(H > 0 && G > 0 && H % G == 0 && dk > 0 && dv > 0 && dv <= 64 * DVU && dk <= 4096);
-    MXH_CHECK(ldq >= H * dk && ldo >= H * dv && chunk >= 0 && window >= 0 && H <= 65535);
-    MXH_CHECK(cu_q || n_rows == n_seqs);
-    const dim3 grid(n_rows, H);
+    MXH_CHECK(ldq >= H * dk && ldo >= H * dv && chunk >= 0 && window >= 0 && H <= 65535 && row_off >= 0);
+    MXH_CHECK(cu_q || (row_off == 0 && n_rows == n_seqs));
+    MXH_CHECK(parts >= 1 && parts <= 65535 && (parts == 1 || (!cu_q && part_len > 0 && part_ml && part_o)));
+    const dim3 grid(n_rows, H, parts);
     const size_t sh = (size_t)(dk + 64 + 2) * sizeof(float) + 64 * sizeof(long);
 #define GO(B, O)                                                                                                    \
     attn_rows_kernel<B, O><<<grid, 64, sh, st>>>(q, ldq, kc, vc, bs, bt, bt_stride, cu_q, ctx, n_seqs, row_base, out, \
-                                                 ldo, H, G, dk, dv, scale, chunk, window, sink, out_scale)
+                                                 ldo, H, G, dk, dv, scale, chunk, window, sink, out_scale, row_off,  \
+                                                 parts, part_len, part_ml, part_o)
     if (q16 && o16) GO(true, true);
     else if (q16) GO(true, false);
     else if (o16) GO(false, true);
     else GO(false, false);
 #undef GO
+    if (parts > 1) {
+        const dim3 g2(n_rows, H);
+        if (o16) attn_merge_kernel<true><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, row_base, out, ldo);
+        else attn_merge_kernel<false><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, row_base, out, ldo);
+    }
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_kv_gather(const void* kc, const void* vc, int is16, int bs, const int* table, int lo, int n, int G,
+                             int dk, int dv, void* kh, void* vh, hipStream_t st) {
+    if (n <= 0) return 0;
+    MXH_CHECK(kc && vc && table && kh && vh && bs > 0 && lo >= 0 && G > 0 && G <= 65535 && dk > 0 && dv > 0);
+    const dim3 grid(n, G);
+    if (is16) kv_gather_kernel<bf16_t><<<grid, 64, 0, st>>>((const bf16_t*)kc, (const bf16_t*)vc, bs, table, lo, n, G, dk,
+                                                           dv, (bf16_t*)kh, (bf16_t*)vh);
+    else kv_gather_kernel<float><<<grid, 64, 0, st>>>((const float*)kc, (const float*)vc, bs, table, lo, n, G, dk, dv,
+                                                      (float*)kh, (float*)vh);
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_head_transpose(const void* src, int s16, long s_si, long s_sh, void* dst, int d16, long d_si,
+                                  long d_sh, int n, int H, int d, float scale, hipStream_t st) {
+    if (n <= 0) return 0;
+    MXH_CHECK(src && dst && H > 0 && H <= 65535 && d > 0);
+    const dim3 grid(n, H);
+#define GO(S, D) head_transpose_kernel<S, D><<<grid, 64, 0, st>>>(src, s_si, s_sh, dst, d_si, d_sh, d, scale)
+    if (s16 && d16) GO(true, true);
+    else if (s16) GO(true, false);
+    else if (d16) GO(false, true);
+    else GO(false, false);
+#undef GO
+    return (int)hipGetLastError();
+}
+
+extern "C" int mxh_masked_softmax(const float* sc, void* pw, int p16, long rows, int n, int nk, int p0, int key0,
+                                  float scale, int chunk, int window, int sink, hipStream_t st) {
+    if (rows <= 0) return 0;
+    MXH_CHECK(sc && pw && n > 0 && nk > 0 && rows % n == 0 && rows < (1L << 31) && key0 >= 0 && p0 >= key0);
+    if (p16) masked_softmax_kernel<true><<<(unsigned)rows, 256, 0, st>>>(sc, pw, n, nk, p0, key0, scale, chunk, window, sink);
+    else masked_softmax_kernel<false><<<(unsigned)rows, 256, 0, st>>>(sc, pw, n, nk, p0, key0, scale, chunk, window, sink);
     return (int)hipGetLastError();
 }

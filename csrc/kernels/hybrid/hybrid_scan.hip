@@ -37,58 +37,86 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
     const bool fresh = positions[row0] == 0 || slot < 0;
     const bool live = col < P;
     const int g = h / (H / G);
-    float* sp = state + (((long)(slot < 0 ? 0 : slot) * H + h) * N + part * NPL) * P + col;
+    // addresses are clamped so that every load below is unconditional (all in flight together); what a lane must not
+    // use is replaced by zero afterwards
+    const int colc = min(col, P - 1);
+    float* sp = state + (((long)(slot < 0 ? 0 : slot) * H + h) * N) * P + colc;
     float S[NPL];
 #pragma unroll
-    for (int j = 0; j < NPL; ++j) S[j] = (!fresh && live && part * NPL + j < N) ? sp[(long)j * P] : 0.f;
+    for (int j = 0; j < NPL; ++j) {
+        const int e = part * NPL + j;
+        const float x = sp[(long)min(e, N - 1) * P];
+        S[j] = (!fresh && live && e < N) ? x : 0.f;
+    }
     const float* kp = k + (long)g * N;
     const float* qp = q + (long)g * N;
     const float sk = skip ? skip[h] : 0.f;
     for (int i = threadIdx.x; i < 2 * NP; i += blockDim.x) {
         const int w = i / NP, e = i % NP;
-        kq[0][w][e] = e < N ? (w ? qp[(long)row0 * ldq + e] : kp[(long)row0 * ldk + e]) : 0.f;
+        const float x = w ? qp[(long)row0 * ldq + min(e, N - 1)] : kp[(long)row0 * ldk + min(e, N - 1)];
+        kq[0][w][e] = e < N ? x : 0.f;
     }
+    const float* vp = v + (long)h * P + colc;
+    const float* ap = decay + h;
+    const float* cp = coef + h;
+    // the next token's decay, write strength and value are requested one step ahead of their use
+    float a_n = ap[(long)row0 * H], c_n = cp[(long)row0 * H], v_n = vp[(long)row0 * ldv];
     for (int t = 0; t < n; ++t) {
         const int row = row0 + t, b = t & 1;
+        const float a = a_n, c = c_n, vv = live ? v_n : 0.f;
         __syncthreads();
         if (t + 1 < n) {
             for (int i = threadIdx.x; i < 2 * NP; i += blockDim.x) {
                 const int w = i / NP, e = i % NP;
-                kq[b ^ 1][w][e] = e < N ? (w ? qp[(long)(row + 1) * ldq + e] : kp[(long)(row + 1) * ldk + e]) : 0.f;
+                const float x = w ? qp[(long)(row + 1) * ldq + min(e, N - 1)] : kp[(long)(row + 1) * ldk + min(e, N - 1)];
+                kq[b ^ 1][w][e] = e < N ? x : 0.f;
             }
+            a_n = ap[(long)(row + 1) * H];
+            c_n = cp[(long)(row + 1) * H];
+            v_n = vp[(long)(row + 1) * ldv];
         }
-        const float a = decay[(long)row * H + h], c = coef[(long)row * H + h];
-        const float vv = live ? v[(long)row * ldv + (long)h * P + col] : 0.f;
         const float* kb = &kq[b][0][part * NPL];
         const float* qb = &kq[b][1][part * NPL];
         float u;
         if constexpr (DELTA) {
-            float d = 0.f;
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;  // four chains instead of one of NPL dependent adds
 #pragma unroll
-            for (int j = 0; j < NPL; ++j) {
+            for (int j = 0; j < NPL; j += 4) {
                 S[j] *= a;
-                d += S[j] * kb[j];
+                S[j + 1] *= a;
+                S[j + 2] *= a;
+                S[j + 3] *= a;
+                d0 += S[j] * kb[j];
+                d1 += S[j + 1] * kb[j + 1];
+                d2 += S[j + 2] * kb[j + 2];
+                d3 += S[j + 3] * kb[j + 3];
             }
-            d = group_sum<LPC>(d);
+            const float d = group_sum<LPC>((d0 + d1) + (d2 + d3));
             u = c * (vv - d);
         } else {
 #pragma unroll
             for (int j = 0; j < NPL; ++j) S[j] *= a;
             u = c * vv;
         }
-        float o = 0.f;
+        float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
-        for (int j = 0; j < NPL; ++j) {
+        for (int j = 0; j < NPL; j += 4) {
             S[j] += kb[j] * u;
-            o += S[j] * qb[j];
+            S[j + 1] += kb[j + 1] * u;
+            S[j + 2] += kb[j + 2] * u;
+            S[j + 3] += kb[j + 3] * u;
+            o0 += S[j] * qb[j];
+            o1 += S[j + 1] * qb[j + 1];
+            o2 += S[j + 2] * qb[j + 2];
+            o3 += S[j + 3] * qb[j + 3];
         }
-        o = group_sum<LPC>(o);
+        const float o = group_sum<LPC>((o0 + o1) + (o2 + o3));
         if (live && part == 0) out[(long)row * ldo + (long)h * P + col] = o + sk * vv;
     }
     if (slot >= 0 && live) {
 #pragma unroll
         for (int j = 0; j < NPL; ++j)
-            if (part * NPL + j < N) sp[(long)j * P] = S[j];
+            if (part * NPL + j < N) sp[(long)(part * NPL + j) * P] = S[j];
     }
 }
 

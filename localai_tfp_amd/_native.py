@@ -150,8 +150,14 @@ HYBRID_SIGS = {
     # T, stream
     "mxh_rope_norm_append": [P, P, P, I, I, I, P, I, I, I, I, I, F, I, F, P, I, I, P, P, I, P, I, P],
     # q, ldq, q16, kc, vc, bs, bt, bt_stride, cu_q, ctx, n_seqs, n_rows, row_base, out, ldo, o16, H, G, dk, dv, scale,
-    # chunk, window, sink, out_scale, stream
-    "mxh_attention": [P, I, I, P, P, I, P, I, P, P, I, I, I, P, I, I, I, I, I, I, F, I, I, I, F, P],
+    # chunk, window, sink, out_scale, row_off, parts, part_len, part_ml, part_o, stream
+    "mxh_attention": [P, I, I, P, P, I, P, I, P, P, I, I, I, P, I, I, I, I, I, I, F, I, I, I, F, I, I, I, P, P, P],
+    # kc, vc, is16, bs, table, lo, n, G, dk, dv, kh, vh, stream
+    "mxh_kv_gather": [P, P, I, I, P, I, I, I, I, I, P, P, P],
+    # src, s16, s_stride_i, s_stride_h, dst, d16, d_stride_i, d_stride_h, n, H, d, scale, stream
+    "mxh_head_transpose": [P, I, L, L, P, I, L, L, I, I, I, F, P],
+    # scores, weights, w16, rows, n, nk, p0, key0, scale, chunk, window, sink, stream
+    "mxh_masked_softmax": [P, P, I, L, I, I, I, I, F, I, I, I, P],
     # x, ldx, w, bias, taps, silu, tails, state, positions, n_dec, pf_cu, n_pf, out, ldo, T, C, stream
     "mxh_causal_conv": [P, I, P, P, I, I, P, P, P, I, P, I, P, I, I, I, P],
     # x, ldx, heads, dim, eps, scale, T, stream

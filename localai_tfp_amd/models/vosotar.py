@@ -33,6 +33,7 @@ import torch
 
 from ..ops import latent as LA
 from ..ops.dense import Dense
+from ..ops.dense import bmm_f32 as _bmm_f32
 
 ARCH = "Vosotar"
 
@@ -394,27 +395,6 @@ class VosotarModel:
                 return hs.float()
             self.last_hidden = hs.float()
         return self.head.into(hs, ws.logits[:S])
-
-
-_BMM_OUT_DTYPE: dict = {}
-
-
-def _bmm_f32(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out (fp32) = a @ b batched; 16-bit operands keep the fp32 accumulator where the library exposes it."""
-    if a.dtype == torch.float32:
-        return torch.bmm(a, b, out=out)
-    ok = _BMM_OUT_DTYPE.get(a.dtype)
-    if ok is None:
-        try:
-            torch.bmm(a[:, :1], b, out_dtype=torch.float32)
-            ok = True
-        except Exception:
-            ok = False
-        _BMM_OUT_DTYPE[a.dtype] = ok
-    if ok:
-        return torch.bmm(a, b, out_dtype=torch.float32, out=out)
-    out.copy_(torch.bmm(a, b))
-    return out
 
 
 # ------------------------------------------------------------------------------------------------ sources

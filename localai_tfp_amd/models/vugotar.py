@@ -289,7 +289,7 @@ class VugotarWeights:
 class VugotarWorkspace:
     """Step scratch sized for the largest step; forward() only takes views (static addresses for graph capture)."""
 
-    def __init__(self, model: "VugotarModel", max_tokens: int, max_seqs: int, logits_rows: int):
+    def __init__(self, model: "VugotarModel", max_tokens: int, max_seqs: int, logits_rows: int, max_parts: int = 16):
         cfg, dev, md = model.cfg, model.device, model.dtype
         T, C = max_tokens, cfg.hidden
         f32 = dict(dtype=torch.float32, device=dev)
@@ -323,6 +323,12 @@ class VugotarWorkspace:
         self.route = torch.empty((T * n_e,), **f32)
         self.hs = torch.empty((S, C), **m16)
         self.logits = torch.empty((S, cfg.vocab), **f32)
+        # partial results of decode rows whose visible keys are split into partitions
+        h_att = max([L.mixer.left.heads for L in cfg.layers if L.type == "parallel"] or [1])
+        v_att = max([L.mixer.left.vdim for L in cfg.layers if L.type == "parallel"] or [1])
+        rows = max_seqs * h_att * max(1, min(max_parts, 64))
+        self.part_ml = torch.empty((rows, 2), **f32)
+        self.part_o = torch.empty((rows, v_att), **f32)
 
 
 class VugotarModel:
@@ -372,7 +378,7 @@ class VugotarModel:
         return [sum(e["kv"]) for e in self.cache_spec() if e.get("kv")]
 
     def make_workspace(self, max_tokens: int, max_seqs: int, logits_rows: int = 0, max_parts: int = 64):
-        return VugotarWorkspace(self, max_tokens, max_seqs, logits_rows)
+        return VugotarWorkspace(self, max_tokens, max_seqs, logits_rows, max_parts)
 
     def weight_bytes(self) -> int:
         n = self.embed.numel() * self.embed.element_size() + self.head.w.numel() * self.head.w.element_size()
@@ -535,7 +541,7 @@ class VugotarModel:
                             y[:, c["lv"]:c["lv"] + G * dv], fb.positions, H, G, dk, dv, a.rot_dims, a.rot_base, True,
                             eps, q, kv[0], kv[1], fb.slots)
         HY.masked_attention(q, kv[0], kv[1], rag, H, G, dk, dv, a.scale, cat[:, :H * dv], chunk=a.chunk, sink=True,
-                            out_scale=mx.left_scale)
+                            out_scale=mx.left_scale, workspace=(ws.part_ml, ws.part_o))
         return H * dv
 
     def _right(self, mx: ParallelCfg, W, y, c, rag, state, tails, ws, cat, k0: int, eps) -> int:

@@ -97,6 +97,31 @@ class Dense:
         return acc
 
 
+_BMM_OUT_DTYPE: dict = {}
+
+
+def bmm_f32(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 batched product a @ b; 16-bit operands keep the fp32 accumulator where the library exposes it."""
+    if a.dtype == torch.float32:
+        return torch.bmm(a, b, out=out) if out is not None else torch.bmm(a, b)
+    ok = _BMM_OUT_DTYPE.get(a.dtype)
+    if ok is None:
+        try:
+            torch.bmm(a[:1, :1], b[:1], out_dtype=torch.float32)
+            ok = True
+        except Exception:
+            ok = False
+        _BMM_OUT_DTYPE[a.dtype] = ok
+    if ok:
+        return torch.bmm(a, b, out_dtype=torch.float32, out=out) if out is not None else \
+            torch.bmm(a, b, out_dtype=torch.float32)
+    r = torch.bmm(a, b).float()
+    if out is not None:
+        out.copy_(r)
+        return out
+    return r
+
+
 def layernorm(x: torch.Tensor, w, b, eps: float, out_dtype) -> torch.Tensor:
     """fp32 [M, H] -> layer-normed in out_dtype (norm.hip on GPU)."""
     from . import core as K

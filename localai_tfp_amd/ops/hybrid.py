@@ -141,14 +141,78 @@ def _attn_ref(q, kc, vc, table, ctx, pos0, H, G, dk, dv, scale, chunk, window, s
     out.copy_((o.reshape(n, H * dv) * out_scale).to(out.dtype))
 
 
+GEMM_MIN_ROWS = 64  # prompt chunks of at least this many rows take the library-GEMM route (GPU)
+GEMM_MAX_SCORES = 1 << 26  # fp32 scores of one sub-problem of that route
+DECODE_WAVES = 4096  # decode rows: waves to aim for when splitting contexts into key partitions
+
+
+def decode_part_len(n_dec: int, heads: int, visible: int) -> int:
+    """Keys per partition of the decode rows: one wave walks a (row, head, partition), so few sequences with long
+    visible ranges are split finely (down to two 64-key tiles) and large batches coarsely."""
+    want = max(1, DECODE_WAVES // max(1, n_dec * heads))
+    per = -(-max(1, visible) // want)
+    return max(128, -(-per // 64) * 64)
+
+
+def _visible_blocks(p0: int, n: int, chunk: int, window: int, heads: int):
+    """Sub-problems (first row position, end row position, first key position) of a chunk of n rows starting at
+    position p0: rows of one mask chunk share their first key; every block's fp32 scores stay within
+    GEMM_MAX_SCORES."""
+    out = []
+    if chunk:
+        spans = [(max(p0, c * chunk), min(p0 + n, (c + 1) * chunk), c * chunk)
+                 for c in range(p0 // chunk, (p0 + n - 1) // chunk + 1)]
+    else:
+        spans = [(p0, p0 + n, None)]
+    for a, b, key0 in spans:
+        k0 = key0 if key0 is not None else 0
+        rows = max(GEMM_MIN_ROWS, GEMM_MAX_SCORES // max(1, heads * (b - k0)))
+        for a2 in range(a, b, rows):
+            b2 = min(b, a2 + rows)
+            out.append((a2, b2, key0 if key0 is not None else max(0, a2 - window + 1) if window else 0))
+    return out
+
+
+def _attn_gemm_chunk(q, kc, vc, table, p0, n, H, G, dk, dv, scale, chunk, window, sink, out, out_scale):
+    """A long prompt chunk (rows q [n, H*dk] at positions p0 ..) as library GEMMs: per block of rows, the visible keys
+    and values are gathered head-major from the pages, scores = Q K^T (fp32), masked sink softmax, out = P V (fp32)."""
+    from .dense import bmm_f32
+    st = N.stream_ptr()
+    md, dev, rep, bs = q.dtype, q.device, H // G, kc.shape[1]
+    i16 = _is16(q)
+    for a, b, key0 in _visible_blocks(p0, n, chunk, window, H):
+        n2, nk = b - a, b - key0
+        kh = torch.empty((G, nk, dk), dtype=md, device=dev)
+        vh = torch.empty((G, nk, dv), dtype=md, device=dev)
+        N.kcall("mxh_kv_gather", kc.data_ptr(), vc.data_ptr(), i16, bs, table.data_ptr(), key0, nk, G, dk, dv,
+                kh.data_ptr(), vh.data_ptr(), st)
+        qh = torch.empty((H, n2, dk), dtype=md, device=dev)
+        qr = q[a - p0:]
+        N.kcall("mxh_head_transpose", qr.data_ptr(), i16, qr.stride(0), dk, qh.data_ptr(), i16, dk, n2 * dk, n2, H, dk,
+                1.0, st)
+        sc = bmm_f32(qh.view(G, rep * n2, dk), kh.transpose(1, 2))
+        pw = torch.empty((G, rep * n2, nk), dtype=md, device=dev)
+        N.kcall("mxh_masked_softmax", sc.data_ptr(), pw.data_ptr(), i16, H * n2, n2, nk, a, key0, float(scale),
+                int(chunk), int(window), int(sink), st)
+        o = bmm_f32(pw, vh)
+        orow = out[a - p0:]
+        N.kcall("mxh_head_transpose", o.data_ptr(), 0, dv, n2 * dv, orow.data_ptr(), _is16(out), orow.stride(0), dv, n2,
+                H, dv, float(out_scale), st)
+
+
 def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: Ragged, H: int, G: int, dk: int, dv: int,
                      scale: float, out: torch.Tensor, chunk: int = 0, window: int = 0, sink: bool = False,
-                     out_scale: float = 1.0):
+                     out_scale: float = 1.0, workspace=None):
     """Causal attention of q [T, H*dk] over the paged pools (rope_norm_append's layout); query head h reads key /
     value head h // (H / G). The row at position i sees j in [lo, i]: lo = (i // chunk) * chunk with `chunk`,
     max(0, i - window + 1) with `window`, else 0. `sink` adds exp(0) to the softmax denominator. out [T, H*dv]
     (may be a column slice; fp32 or bf16) receives out_scale times the result. q, pools and out share fp32 or bf16
-    operands; scores, softmax and the accumulators are fp32."""
+    operands; scores, softmax and the accumulators are fp32.
+
+    On the GPU decode rows and short chunks run the row kernel (one wave per row and head; decode rows split their
+    visible keys into partitions merged through `workspace` = (fp32 [rows, 2], fp32 [rows, dv]), rows >= n_dec * H
+    * partitions); chunks of GEMM_MIN_ROWS rows and more, when the step's chunk sizes are known on the host, run as
+    library GEMMs around a masked softmax kernel."""
     T = q.shape[0]
     if T == 0:
         return out
@@ -176,13 +240,44 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
     st = N.stream_ptr()
     common = (H, G, dk, dv, float(scale), int(chunk), int(window), int(sink), float(out_scale))
     if nd:
+        vis = rag.dec_max_len
+        vis = min(vis, chunk) if chunk else min(vis, window) if window else vis
+        parts, plen = 1, 0
+        if workspace is not None:
+            plen = decode_part_len(nd, H, vis)
+            parts = -(-vis // plen)
+            room = workspace[0].shape[0] // (nd * H)
+            if parts > room:
+                parts = max(1, room)
+                plen = -(-(-(-vis // parts)) // 64) * 64
+        ml, po = (workspace[0], workspace[1]) if parts > 1 else (None, None)
         N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
                 rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), None, rag.dec_lens.data_ptr(), nd, nd, 0,
-                out.data_ptr(), out.stride(0), _is16(out), *common, st)
+                out.data_ptr(), out.stride(0), _is16(out), *common, 0, parts, plen if parts > 1 else 0, N.ptr(ml),
+                N.ptr(po), st)
     if rag.n_pf:
-        N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
-                rag.pf_bt.data_ptr(), rag.pf_bt.stride(0), rag.pf_cu.data_ptr(), rag.pf_ctx.data_ptr(), rag.n_pf,
-                T - nd, nd, out.data_ptr(), out.stride(0), _is16(out), *common, st)
+        lens = rag.pf_q_host if len(rag.pf_q_host) == rag.n_pf and len(rag.pf_ctx_host) == rag.n_pf else None
+
+        def rows_kernel(row_off, n_rows):
+            N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
+                    rag.pf_bt.data_ptr(), rag.pf_bt.stride(0), rag.pf_cu.data_ptr(), rag.pf_ctx.data_ptr(), rag.n_pf,
+                    n_rows, nd, out.data_ptr(), out.stride(0), _is16(out), *common, row_off, 1, 0, None, None, st)
+        if lens is None or max(lens) < GEMM_MIN_ROWS:
+            rows_kernel(0, T - nd)
+            return out
+        r, run0 = 0, None  # run0: first row of a run of consecutive short chunks
+        for k, n in enumerate(lens):
+            if n >= GEMM_MIN_ROWS:
+                if run0 is not None:
+                    rows_kernel(run0, r - run0)
+                    run0 = None
+                _attn_gemm_chunk(q[nd + r:nd + r + n], kc, vc, rag.pf_bt[k], rag.pf_ctx_host[k] - n, n, H, G, dk, dv,
+                                 scale, chunk, window, sink, out[nd + r:nd + r + n], out_scale)
+            elif n and run0 is None:
+                run0 = r
+            r += n
+        if run0 is not None:
+            rows_kernel(run0, r - run0)
     return out
 
 

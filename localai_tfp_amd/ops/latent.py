@@ -35,6 +35,9 @@ class Ragged:
         self.dec_bt, self.dec_lens = fb.dec_block_tables, fb.dec_seq_lens
         self.pf_bt, self.pf_ctx = fb.pf_block_tables, fb.pf_ctx_lens
         self.dec_max_len = fb.dec_max_len
+        # rows and context length of each chunk on the host (empty when the step replays a captured graph)
+        self.pf_q_host = list(getattr(fb, "pf_q_lens_host", None) or [])
+        self.pf_ctx_host = list(getattr(fb, "pf_ctx_lens_host", None) or [])
 
     def host_segments(self):
         """[(first row, rows, index into `state`)] on the host."""

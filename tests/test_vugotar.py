@@ -113,6 +113,7 @@ class _FB:
         self.pf_block_tables = None if pf_bt is None else torch.tensor(pf_bt, **i32)
         self.pf_ctx_lens = None if pf_ctx is None else torch.tensor(pf_ctx, **i32)
         self.dec_max_len = max(dec_lens) if dec_lens else 0
+        self.pf_q_lens_host, self.pf_ctx_lens_host = list(chunks), list(pf_ctx or [])
 
 
 def steps_of(n, cuts):
@@ -180,6 +181,7 @@ def _attention_case(dev, dt, H, G, dk, dv, rot, chunk, n, cuts, bs, scale, plant
     vc = torch.full((nb + 3, bs, G * dv), -5.0, dtype=md, device=dev)
     wide = torch.cat([torch.randn(n, 3, generator=g), q, k, v], 1).to(dev)  # the projections as column slices
     got = torch.empty(n, H * dv + 5, device=dev, dtype=md)
+    part = (torch.empty(H * 8, 2, device=dev), torch.empty(H * 8, dv, device=dev))  # room for eight partitions
     for n_dec, chunks, at in steps_of(n, cuts):
         c = 1 if n_dec else chunks[0]
         rows = list(range(at, at + c))
@@ -192,15 +194,18 @@ def _attention_case(dev, dt, H, G, dk, dv, rot, chunk, n, cuts, bs, scale, plant
         HY.rope_norm_append(w[:, 3:3 + H * dk], w[:, 3 + H * dk:3 + (H + G) * dk], w[:, 3 + (H + G) * dk:],
                             fb.positions, H, G, dk, dv, rot, base, True, eps, qo, kc, vc, fb.slots)
         HY.masked_attention(qo, kc, vc, HY.Ragged(fb), H, G, dk, dv, scale, got[at:at + c, 5:], chunk=chunk, sink=True,
-                            out_scale=0.5)
+                            out_scale=0.5, workspace=part)
     return got[:, 5:].float() * 2, want
 
 
 @pytest.mark.parametrize("dev,dt,tol", RUNS)
-def test_attention_chunk_edges_pages_and_sink(dev, dt, tol):
+@pytest.mark.parametrize("gemm_rows", [64, 8])
+def test_attention_chunk_edges_pages_and_sink(dev, dt, tol, gemm_rows, monkeypatch):
     """Planted keys carry nearly all the weight: the first key of the query's chunk (just inside), the last key of
     the chunk before (just outside: the output must not move towards it), a key across a page border, the query's own
-    position; in prompt portions and in rows decoded alone."""
+    position; in prompt portions and in rows decoded alone. On the GPU portions of `gemm_rows` rows and more take
+    the library-GEMM route, shorter ones and decoded rows the row kernel."""
+    monkeypatch.setattr(HY, "GEMM_MIN_ROWS", gemm_rows)
     chunk, bs, n = 40, 16, 150
     plant = [(79, 40), (119, 80), (120, 119), (121, 120), (95, 81), (149, 127), (60, 60), (39, 0), (41, 39)]
     for cuts in ([n], [37, 2, 41, 1, 1, 38, 1, 1, 1, 27], [118] + [1] * 32):
@@ -211,6 +216,10 @@ def test_attention_chunk_edges_pages_and_sink(dev, dt, tol):
     close(got, want, tol)
     got, want = _attention_case(dev, dt, 2, 2, 64, 72, 64, 0, 90, [50, 40], 8, 0.3)  # no chunks: plain causal
     close(got, want, tol)
+    # rows decoded alone behind 260 and more visible keys: their keys are split into partitions and merged
+    plant = [(270, 3), (280, 127), (281, 128), (299, 255), (290, 256), (295, 295)]
+    got, want = _attention_case(dev, dt, 2, 1, 16, 16, 16, 0, 300, [200, 60] + [1] * 40, 16, 3.0, plant)
+    close(got, want, tol * (4 if dt == "bfloat16" else 1))
 
 
 @pytest.mark.parametrize("dev", DEVS)
