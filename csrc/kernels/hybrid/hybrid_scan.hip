@@ -1,26 +1,54 @@
 // hybrid_scan.hip: the linear recurrence of gated-delta-rule and state-space (duality form) layers (ops/hybrid.py
 // state_scan). Per sequence and head, over the step's rows in order:
 //     S <- a_t S;   u = c_t (v_t - S^T k_t)  [delta]   or   u = c_t v_t;   S <- S + k_t u^T;   o_t = S^T q_t (+ D v_t)
-// S is [N, P] fp32. Its P columns never mix, so a column belongs to LPC neighbouring lanes that each keep NPL of its
-// N numbers in registers for the whole chunk; the two dot products of a step are finished with LPC-wide shuffles. k_t
-// and q_t are the same for every column of a head: the block stages them in LDS (double buffered, one barrier per
-// token). The state is read from the sequence's slot unless the chunk starts at position 0, and written back after
-// the chunk's last row: a decode row is a chunk of one, a prompt chunk walks its rows inside one launch.
+// S has N numbers for each of the head's P value columns, fp32, stored column-major: state [slots, H, P, N]. The
+// columns never mix, so a column belongs to LPC neighbouring lanes (4, or the 16 of one DPP row) that each keep NPL
+// consecutive numbers of it in registers for the whole chunk: a step costs 4 NPL vector operations and two LPC-wide
+// sums done with DPP moves, and a lane's part of the state is one contiguous run in memory (a column's lanes read N
+// contiguous floats, a wave's columns are adjacent). k_t and q_t are the same for every column of a head: the block
+// stages them in LDS together with the tokens' decays, write strengths and values, 8 or 16 tokens at a time in two
+// buffers; the next tokens' numbers are requested from memory before the current ones are worked on and wait in
+// registers meanwhile, so memory latency and the barrier are paid once per 8 or 16 steps. The state is read from the
+// sequence's slot unless the chunk starts at position 0, and written back after the chunk's last row: a decode row is
+// a chunk of one, a prompt chunk walks its rows inside one launch.
 #include "../mx_common.h"
 
 namespace {
 
-// grid (column blocks, H, sequences); block = cols * LPC threads (a multiple of 64)
+template <int CTRL>
+MX_DEV float dpp_add(float v) {
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+// sum over the LPC (4 or 16) neighbouring lanes of a column, returned to each of them
+template <int LPC>
+MX_DEV float lanes_sum(float v) {
+    v = dpp_add<0xB1>(v);  // quad_perm [1, 0, 3, 2]
+    v = dpp_add<0x4E>(v);  // quad_perm [2, 3, 0, 1]
+    if constexpr (LPC == 16) {
+        v = dpp_add<0x124>(v);  // row_ror 4
+        v = dpp_add<0x128>(v);  // row_ror 8
+    }
+    return v;
+}
+
+// grid (column blocks, H, sequences); block = 256 threads = 256 / LPC columns
 template <int NPL, int LPC, bool DELTA>
 __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk, const float* q, int ldq,
                                                          const float* v, int ldv, const float* decay, const float* coef,
                                                          const float* skip, float* state, const int* seq_state,
                                                          const int* positions, int n_dec, const int* pf_cu, float* out,
                                                          int ldo, int H, int G, int N, int P) {
+    static_assert(LPC == 4 || LPC == 16, "a column's lanes are a quad or a DPP row");
+    constexpr int NT = 256;
     constexpr int NP = NPL * LPC;  // padded N
-    __shared__ float kq[2][2][NP];
-    const int cols = blockDim.x / LPC;
-    const int col = blockIdx.x * cols + threadIdx.x / LPC;
+    constexpr int COLS = NT / LPC;
+    constexpr int TB = NP <= 128 ? 16 : 8;  // tokens staged together
+    constexpr int KQ_PT = TB * 2 * NP / NT, V_PT = (TB * COLS + NT - 1) / NT;
+    __shared__ float kq[2][TB][2][NP];
+    __shared__ float vs[2][TB][COLS];
+    __shared__ float ac[2][TB][2];
+    const int cl = threadIdx.x / LPC;
+    const int col = blockIdx.x * COLS + cl;
     const int part = threadIdx.x % LPC;
     const int h = blockIdx.y, s = blockIdx.z;
     int row0, n;
@@ -40,83 +68,118 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
     // addresses are clamped so that every load below is unconditional (all in flight together); what a lane must not
     // use is replaced by zero afterwards
     const int colc = min(col, P - 1);
-    float* sp = state + (((long)(slot < 0 ? 0 : slot) * H + h) * N) * P + colc;
+    float* sp = state + (((long)(slot < 0 ? 0 : slot) * H + h) * P + colc) * N;
+    const bool whole = N == NP && (N & 3) == 0;  // no padding: a lane's run is NPL aligned floats
     float S[NPL];
+    if (whole) {
+        const float4* s4 = (const float4*)(sp + part * NPL);
 #pragma unroll
-    for (int j = 0; j < NPL; ++j) {
-        const int e = part * NPL + j;
-        const float x = sp[(long)min(e, N - 1) * P];
-        S[j] = (!fresh && live && e < N) ? x : 0.f;
+        for (int j = 0; j < NPL / 4; ++j) {
+            const float4 x = s4[j];
+            S[4 * j] = x.x;
+            S[4 * j + 1] = x.y;
+            S[4 * j + 2] = x.z;
+            S[4 * j + 3] = x.w;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) S[j] = sp[min(part * NPL + j, N - 1)];
     }
+    const bool keep = !fresh && live;
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) S[j] = (keep && part * NPL + j < N) ? S[j] : 0.f;
     const float* kp = k + (long)g * N;
     const float* qp = q + (long)g * N;
     const float sk = skip ? skip[h] : 0.f;
-    for (int i = threadIdx.x; i < 2 * NP; i += blockDim.x) {
-        const int w = i / NP, e = i % NP;
-        const float x = w ? qp[(long)row0 * ldq + min(e, N - 1)] : kp[(long)row0 * ldk + min(e, N - 1)];
-        kq[0][w][e] = e < N ? x : 0.f;
-    }
-    const float* vp = v + (long)h * P + colc;
-    const float* ap = decay + h;
-    const float* cp = coef + h;
-    // the next token's decay, write strength and value are requested one step ahead of their use
-    float a_n = ap[(long)row0 * H], c_n = cp[(long)row0 * H], v_n = vp[(long)row0 * ldv];
-    for (int t = 0; t < n; ++t) {
-        const int row = row0 + t, b = t & 1;
-        const float a = a_n, c = c_n, vv = live ? v_n : 0.f;
+    const int last = row0 + n - 1;
+    // TB tokens' k, q, value, decay and write strength wait in registers while the TB tokens before them are worked
+    // on, then move to LDS: memory latency is paid once per TB steps, and a barrier too
+    float st_kq[KQ_PT], st_v[V_PT], st_ac = 0.f;
+    auto fetch = [&](int c) {
+        const int r0 = row0 + c * TB;
+#pragma unroll
+        for (int i = 0; i < KQ_PT; ++i) {
+            const int idx = threadIdx.x + i * NT;
+            const int tt = idx / (2 * NP), w = (idx / NP) & 1, e = idx % NP;
+            const long row = min(r0 + tt, last);
+            const float x = w ? qp[row * ldq + min(e, N - 1)] : kp[row * ldk + min(e, N - 1)];
+            st_kq[i] = e < N ? x : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < V_PT; ++i) {
+            const int idx = min(threadIdx.x + i * NT, TB * COLS - 1);
+            const int tt = idx / COLS, cc = idx % COLS;
+            const long row = min(r0 + tt, last);
+            st_v[i] = v[row * ldv + (long)h * P + min((int)blockIdx.x * COLS + cc, P - 1)];
+        }
+        if (threadIdx.x < 2 * TB) {
+            const long row = min(r0 + (int)threadIdx.x / 2, last);
+            st_ac = (threadIdx.x & 1) ? coef[row * H + h] : decay[row * H + h];
+        }
+    };
+    auto publish = [&](int b) {
+#pragma unroll
+        for (int i = 0; i < KQ_PT; ++i) (&kq[b][0][0][0])[threadIdx.x + i * NT] = st_kq[i];
+#pragma unroll
+        for (int i = 0; i < V_PT; ++i)
+            if (threadIdx.x + i * NT < TB * COLS) (&vs[b][0][0])[threadIdx.x + i * NT] = st_v[i];
+        if (threadIdx.x < 2 * TB) (&ac[b][0][0])[threadIdx.x] = st_ac;
+    };
+    const int nchunks = (n + TB - 1) / TB;
+    fetch(0);
+    publish(0);
+    __syncthreads();
+    for (int c = 0; c < nchunks; ++c) {
+        const int b = c & 1;
+        if (c + 1 < nchunks) fetch(c + 1);
+        const int nt = min(TB, n - c * TB);
+        for (int tt = 0; tt < nt; ++tt) {
+            const int row = row0 + c * TB + tt;
+            const float a = ac[b][tt][0], cf = ac[b][tt][1];
+            const float vv = live ? vs[b][tt][cl] : 0.f;
+            const float* kb = &kq[b][tt][0][part * NPL];
+            const float* qb = &kq[b][tt][1][part * NPL];
+            float u;
+            if constexpr (DELTA) {
+                float d0 = 0.f, d1 = 0.f;  // two chains instead of one of NPL dependent adds
+#pragma unroll
+                for (int j = 0; j < NPL; j += 2) {
+                    S[j] *= a;
+                    S[j + 1] *= a;
+                    d0 += S[j] * kb[j];
+                    d1 += S[j + 1] * kb[j + 1];
+                }
+                u = cf * (vv - lanes_sum<LPC>(d0 + d1));
+            } else {
+#pragma unroll
+                for (int j = 0; j < NPL; ++j) S[j] *= a;
+                u = cf * vv;
+            }
+            float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < NPL; j += 2) {
+                S[j] += kb[j] * u;
+                S[j + 1] += kb[j + 1] * u;
+                o0 += S[j] * qb[j];
+                o1 += S[j + 1] * qb[j + 1];
+            }
+            const float o = lanes_sum<LPC>(o0 + o1);
+            if (live && part == 0) out[(long)row * ldo + (long)h * P + col] = o + sk * vv;
+        }
+        // the other buffer was last read while chunk c - 1 was worked on, before the barrier that ended that round
+        if (c + 1 < nchunks) publish(b ^ 1);
         __syncthreads();
-        if (t + 1 < n) {
-            for (int i = threadIdx.x; i < 2 * NP; i += blockDim.x) {
-                const int w = i / NP, e = i % NP;
-                const float x = w ? qp[(long)(row + 1) * ldq + min(e, N - 1)] : kp[(long)(row + 1) * ldk + min(e, N - 1)];
-                kq[b ^ 1][w][e] = e < N ? x : 0.f;
-            }
-            a_n = ap[(long)(row + 1) * H];
-            c_n = cp[(long)(row + 1) * H];
-            v_n = vp[(long)(row + 1) * ldv];
-        }
-        const float* kb = &kq[b][0][part * NPL];
-        const float* qb = &kq[b][1][part * NPL];
-        float u;
-        if constexpr (DELTA) {
-            float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;  // four chains instead of one of NPL dependent adds
-#pragma unroll
-            for (int j = 0; j < NPL; j += 4) {
-                S[j] *= a;
-                S[j + 1] *= a;
-                S[j + 2] *= a;
-                S[j + 3] *= a;
-                d0 += S[j] * kb[j];
-                d1 += S[j + 1] * kb[j + 1];
-                d2 += S[j + 2] * kb[j + 2];
-                d3 += S[j + 3] * kb[j + 3];
-            }
-            const float d = group_sum<LPC>((d0 + d1) + (d2 + d3));
-            u = c * (vv - d);
-        } else {
-#pragma unroll
-            for (int j = 0; j < NPL; ++j) S[j] *= a;
-            u = c * vv;
-        }
-        float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
-#pragma unroll
-        for (int j = 0; j < NPL; j += 4) {
-            S[j] += kb[j] * u;
-            S[j + 1] += kb[j + 1] * u;
-            S[j + 2] += kb[j + 2] * u;
-            S[j + 3] += kb[j + 3] * u;
-            o0 += S[j] * qb[j];
-            o1 += S[j + 1] * qb[j + 1];
-            o2 += S[j + 2] * qb[j + 2];
-            o3 += S[j + 3] * qb[j + 3];
-        }
-        const float o = group_sum<LPC>((o0 + o1) + (o2 + o3));
-        if (live && part == 0) out[(long)row * ldo + (long)h * P + col] = o + sk * vv;
     }
     if (slot >= 0 && live) {
+        if (whole) {
+            float4* s4 = (float4*)(sp + part * NPL);
 #pragma unroll
-        for (int j = 0; j < NPL; ++j)
-            if (part * NPL + j < N) sp[(long)(part * NPL + j) * P] = S[j];
+            for (int j = 0; j < NPL / 4; ++j) s4[j] = make_float4(S[4 * j], S[4 * j + 1], S[4 * j + 2], S[4 * j + 3]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NPL; ++j)
+                if (part * NPL + j < N) sp[part * NPL + j] = S[j];
+        }
     }
 }
 
@@ -134,8 +197,8 @@ extern "C" int mxh_state_scan(const float* k, int ldk, const float* q, int ldq, 
     MXH_CHECK(k && q && v && decay && coef && state && seq_state && positions && out && (n_pf == 0 || pf_cu));
     MXH_CHECK(H > 0 && G > 0 && H % G == 0 && N > 0 && N <= 256 && P > 0 && H <= 65535 && n_seqs <= 65535);
     MXH_CHECK(ldk >= G * N && ldq >= G * N && ldv >= H * P && ldo >= H * P);
-    const int lpc = N <= 64 ? 1 : N <= 128 ? 2 : 4;
-    int threads = min(256, ((P * lpc + 63) / 64) * 64);
+    const int lpc = N <= 32 ? 4 : 16;
+    const int threads = 256;
     const int cols = threads / lpc;
     const dim3 grid((P + cols - 1) / cols, H, n_seqs);
 #define GO(NPL, LPC)                                                                                                 \
@@ -149,11 +212,11 @@ extern "C" int mxh_state_scan(const float* k, int ldk, const float* q, int ldq, 
                                                                          state, seq_state, positions, n_dec, pf_cu, \
                                                                          out, ldo, H, G, N, P);                      \
     } while (0)
-    if (N <= 16) GO(16, 1);
-    else if (N <= 32) GO(32, 1);
-    else if (N <= 64) GO(64, 1);
-    else if (N <= 128) GO(64, 2);
-    else GO(64, 4);
+    if (N <= 16) GO(4, 4);
+    else if (N <= 32) GO(8, 4);
+    else if (N <= 64) GO(4, 16);
+    else if (N <= 128) GO(8, 16);
+    else GO(16, 16);
 #undef GO
     return (int)hipGetLastError();
 }

@@ -213,10 +213,11 @@ class HybridCache:
     * `kv[i]`: (keys [num_blocks, block_size, kv_heads * dim], values [.., kv_heads * vdim]) in bf16 or fp32,
       token-major so one append writes one contiguous row, addressed by the block tables and flat slots of the block
       manager; None for runs without attention;
-    * `state[i]`: fp32 [state_slots, heads, N, P] recurrent state, None for runs without a recurrence;
+    * `state[i]`: fp32 [state_slots, heads, P, N] recurrent state (N numbers for each of a head's P value columns),
+      None for runs without a recurrence;
     * `tails[i]`: fp32 [state_slots, taps - 1, channels] last inputs of the run's causal convolution, or None.
 
-    `spec` lists per run a dict with the optional keys "kv": (key row, value row), "state": (heads, N, P),
+    `spec` lists per run a dict with the optional keys "kv": (key row, value row), "state": (heads, P, N),
     "tails": (taps - 1, channels). State slots are handed out per live sequence by `SlotPool`."""
 
     def __init__(self, spec, num_blocks: int, block_size: int, device, dtype=torch.bfloat16, state_slots: int = 0):

@@ -362,10 +362,10 @@ class VugotarModel:
             m = L.mixer
             if L.type == "parallel":
                 a, r = m.left, m.right
-                spec.append({"kv": (a.kv_heads * a.dim, a.kv_heads * a.vdim), "state": (r.heads, r.dim, r.vdim),
+                spec.append({"kv": (a.kv_heads * a.dim, a.kv_heads * a.vdim), "state": (r.heads, r.vdim, r.dim),
                              "tails": (r.conv - 1, 2 * r.kv_heads * r.dim + r.heads * r.vdim)})
             else:
-                spec.append({"state": (m.heads, m.state, m.vdim),
+                spec.append({"state": (m.heads, m.vdim, m.state),
                              "tails": (m.conv - 1, m.inner + 2 * m.groups * m.state)})
         return spec
 

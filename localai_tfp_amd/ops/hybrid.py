@@ -10,7 +10,7 @@
 * `causal_conv`: a per-channel causal convolution over time (optional bias and SiLU) whose last taps-1 inputs are
   carried per sequence;
 * `unit_norm_heads`, `scan_coefs`, `state_scan`: the pieces of a linear recurrence S <- a S + k u^T, o = S^T q per
-  head (S is [N, P], fp32, one per sequence and head). With `delta` the written value is u = c (v - S^T k) after
+  head (S is [N, P], fp32, one per sequence and head, stored column-major). With `delta` the written value is u = c (v - S^T k) after
   the decay (gated delta rule), otherwise u = c v with an optional skip D v on the output (state-space duality form);
 * `gated_group_norm`: unit-RMS norm over groups of columns, a weight, and a SiLU gate before or after the norm;
 * `glu`: silu(a + bias) * (b + bias) with an optional per-row, per-column-group factor (routing weights of experts
@@ -358,8 +358,9 @@ def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.T
         S <- decay_t S;  u = coef_t (v_t - S^T k_t) if delta else coef_t v_t;  S <- S + k_t u^T;
         o_t = S^T q_t (+ skip_h v_t)
     k, q fp32 [T, G*Nk] (head h reads group h // (H / G)), v fp32 [T, H*P], decay / coef fp32 [T, H], out fp32
-    [T, H*P]; all may be column slices. state fp32 [slots, H, Nk, P] is read at the sequence's slot unless its first
-    row is at position 0 (then S starts at zero) and written back after its last row."""
+    [T, H*P]; all may be column slices. state fp32 [slots, H, P, Nk] (a column's Nk numbers are contiguous) is read at
+    the sequence's slot unless its first row is at position 0 (then S starts at zero) and written back after its last
+    row."""
     T = k.shape[0]
     if T == 0:
         return out
@@ -368,7 +369,7 @@ def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.T
         rep = H // G
         for r0, n, si in rag.host_segments():
             slot = st[si]
-            S = torch.zeros(H, Nk, P) if (pos[r0] == 0 or slot < 0) else state[slot].clone()
+            S = torch.zeros(H, Nk, P) if (pos[r0] == 0 or slot < 0) else state[slot].transpose(1, 2).clone()
             for t in range(r0, r0 + n):
                 kt = k[t].float().reshape(G, Nk).repeat_interleave(rep, 0)
                 qt = q[t].float().reshape(G, Nk).repeat_interleave(rep, 0)
@@ -381,13 +382,13 @@ def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.T
                     o = o + skip[:, None] * vt
                 out[t] = o.reshape(H * P)
             if slot >= 0:
-                state[slot] = S
+                state[slot] = S.transpose(1, 2)
         return out
     for t_ in (k, q, v, out):
         _f32c(t_, "state_scan")
-    if tuple(state.shape[1:]) != (H, Nk, P) or not state.is_contiguous() or not decay.is_contiguous() \
+    if tuple(state.shape[1:]) != (H, P, Nk) or not state.is_contiguous() or not decay.is_contiguous() \
             or not coef.is_contiguous() or H % G or Nk > 256:
-        raise ValueError("state_scan: state is [slots, H, N, P] with N <= 256, decay / coef contiguous [T, H]")
+        raise ValueError("state_scan: state is [slots, H, P, N] with N <= 256, decay / coef contiguous [T, H]")
     N.kcall("mxh_state_scan", k.data_ptr(), k.stride(0), q.data_ptr(), q.stride(0), v.data_ptr(), v.stride(0),
             decay.data_ptr(), coef.data_ptr(), N.ptr(skip), state.data_ptr(), rag.state.data_ptr(),
             rag.positions.data_ptr(), rag.n_dec, N.ptr(rag.pf_cu), rag.n_pf, out.data_ptr(), out.stride(0), H, G, Nk,

@@ -301,7 +301,7 @@ def test_state_scan_in_portions(dev, delta, H, G, N, P):
             for t in range(n):
                 S = decay[t, h] * S + coef[t, h] * torch.outer(kk[t], vv[t])
                 want[t, h] = S.T @ qq[t] + skip[h].double() * vv[t]
-    state = torch.full((2, H, N, P), 4.0, device=dev)  # slot 1 is dirty: position 0 must not read it
+    state = torch.full((2, H, P, N), 4.0, device=dev)  # slot 1 is dirty: position 0 must not read it
     out = torch.empty(n, H * P, device=dev)
     dec, cf = torch.empty(n, H, device=dev), torch.empty(n, H, device=dev)
     HY.scan_coefs(a_raw.to(dev), b_raw.to(dev) if delta else None, A_log.to(dev), dtb.to(dev), dec, cf)
