@@ -17,7 +17,7 @@
 
 namespace {
 
-constexpr int DVU = 8;  // value columns per lane: heads of up to 512 numbers
+constexpr int DVU_MAX = 8;  // value columns per lane: heads of up to 512 numbers
 
 template <bool B16>
 MX_DEV float ld1(const void* p, long i) {
@@ -25,49 +25,82 @@ MX_DEV float ld1(const void* p, long i) {
     else return ((const float*)p)[i];
 }
 
-// dot of a pool row with the fp32 query in LDS (n numbers, row and query 16-byte aligned when n % 8 == 0)
-template <bool B16>
-MX_DEV float dot_row(const void* base, long off, const float* q, int n) {
-    float acc = 0.f;
+MX_DEV float dot8(const uint4 w, const float* qq) {
+    return __uint_as_float(w.x << 16) * qq[0] + __uint_as_float(w.x & 0xffff0000u) * qq[1] +
+           __uint_as_float(w.y << 16) * qq[2] + __uint_as_float(w.y & 0xffff0000u) * qq[3] +
+           __uint_as_float(w.z << 16) * qq[4] + __uint_as_float(w.z & 0xffff0000u) * qq[5] +
+           __uint_as_float(w.w << 16) * qq[6] + __uint_as_float(w.w & 0xffff0000u) * qq[7];
+}
+MX_DEV float dot4(const float4 w, const float* qq) { return w.x * qq[0] + w.y * qq[1] + w.z * qq[2] + w.w * qq[3]; }
+
+// dots of one pool row with REP fp32 queries in LDS (q + r * n; n numbers, row and queries 16-byte aligned when
+// n % 8 == 0). Four 16-byte pieces of the row are requested before the first is used: a lane's loads are one
+// dependent chain otherwise. The row is read once for all REP queries.
+template <bool B16, int REP>
+MX_DEV void dot_row(const void* base, long off, const float* q, int n, float (&acc)[REP]) {
+#pragma unroll
+    for (int r = 0; r < REP; ++r) acc[r] = 0.f;
     if ((n & 7) == 0) {
         if constexpr (B16) {
-            const uint4* r = (const uint4*)((const bf16_t*)base + off);
-            for (int i = 0; i < n / 8; ++i) {
-                const uint4 w = r[i];
-                const float* qq = q + i * 8;
-                acc += __uint_as_float(w.x << 16) * qq[0] + __uint_as_float(w.x & 0xffff0000u) * qq[1];
-                acc += __uint_as_float(w.y << 16) * qq[2] + __uint_as_float(w.y & 0xffff0000u) * qq[3];
-                acc += __uint_as_float(w.z << 16) * qq[4] + __uint_as_float(w.z & 0xffff0000u) * qq[5];
-                acc += __uint_as_float(w.w << 16) * qq[6] + __uint_as_float(w.w & 0xffff0000u) * qq[7];
+            const uint4* p = (const uint4*)((const bf16_t*)base + off);
+            const int m = n / 8;
+            int i = 0;
+            for (; i + 4 <= m; i += 4) {
+                const uint4 w0 = p[i], w1 = p[i + 1], w2 = p[i + 2], w3 = p[i + 3];
+#pragma unroll
+                for (int r = 0; r < REP; ++r) {
+                    const float* qq = q + r * n + i * 8;
+                    acc[r] += (dot8(w0, qq) + dot8(w1, qq + 8)) + (dot8(w2, qq + 16) + dot8(w3, qq + 24));
+                }
+            }
+            for (; i < m; ++i) {
+                const uint4 w0 = p[i];
+#pragma unroll
+                for (int r = 0; r < REP; ++r) acc[r] += dot8(w0, q + r * n + i * 8);
             }
         } else {
-            const float4* r = (const float4*)((const float*)base + off);
-            for (int i = 0; i < n / 4; ++i) {
-                const float4 w = r[i];
-                const float* qq = q + i * 4;
-                acc += w.x * qq[0] + w.y * qq[1] + w.z * qq[2] + w.w * qq[3];
+            const float4* p = (const float4*)((const float*)base + off);
+            const int m = n / 4;
+            int i = 0;
+            for (; i + 4 <= m; i += 4) {
+                const float4 w0 = p[i], w1 = p[i + 1], w2 = p[i + 2], w3 = p[i + 3];
+#pragma unroll
+                for (int r = 0; r < REP; ++r) {
+                    const float* qq = q + r * n + i * 4;
+                    acc[r] += (dot4(w0, qq) + dot4(w1, qq + 4)) + (dot4(w2, qq + 8) + dot4(w3, qq + 12));
+                }
+            }
+            for (; i < m; ++i) {
+                const float4 w0 = p[i];
+#pragma unroll
+                for (int r = 0; r < REP; ++r) acc[r] += dot4(w0, q + r * n + i * 4);
             }
         }
-        return acc;
+        return;
     }
-    for (int i = 0; i < n; ++i) acc += ld1<B16>(base, off + i) * q[i];
-    return acc;
+    for (int i = 0; i < n; ++i) {
+        const float w = ld1<B16>(base, off + i);
+#pragma unroll
+        for (int r = 0; r < REP; ++r) acc[r] += w * q[r * n + i];
+    }
 }
 
-// grid (rows, H). cu_q == nullptr: row r is sequence r's single new token at position ctx[r] - 1; otherwise rows are
-// chunks laid end to end, sequence s owning rows [cu_q[s], cu_q[s + 1]) that end at position ctx[s] - 1.
-template <bool B16, bool O16>
+// grid (rows, H / REP, parts): a wave serves the REP query heads h0 .. h0 + REP - 1 of one row, which share a
+// key / value head (REP divides H / G), so keys and values are read once for all of them. cu_q == nullptr: row r is
+// sequence r's single new token at position ctx[r] - 1; otherwise rows are chunks laid end to end, sequence s owning
+// rows [cu_q[s], cu_q[s + 1]) that end at position ctx[s] - 1.
+template <bool B16, bool O16, int REP, int DVU>
 __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, const void* kc, const void* vc, int bs,
                                                        const int* bt, int bt_stride, const int* cu_q, const int* ctx,
                                                        int n_seqs, int row_base, void* out, int ldo, int H, int G,
                                                        int dk, int dv, float scale, int chunk, int window, int sink,
                                                        float out_scale, int row_off, int parts, int part_len,
                                                        float* part_ml, float* part_o) {
-    extern __shared__ float lds[];  // [dk] query, [64] weights, [64] row offsets (as int pairs)
+    extern __shared__ float lds[];  // [REP][dk] queries, [REP][64] weights, [64] row offsets
     float* qs = lds;
-    float* ps = lds + dk;
-    long* rowoff = (long*)(ps + 64 + ((dk & 1) ? 1 : 0));
-    const int r = blockIdx.x + row_off, h = blockIdx.y, lane = threadIdx.x, z = blockIdx.z;
+    float* ps = lds + REP * dk;
+    long* rowoff = (long*)(ps + REP * 64 + ((REP * dk) & 1));
+    const int r = blockIdx.x + row_off, h0 = blockIdx.y * REP, lane = threadIdx.x, z = blockIdx.z;
     int s, pos;
     if (!cu_q) {
         s = r;
@@ -83,9 +116,9 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
         const int n = cu_q[s + 1] - cu_q[s];
         pos = ctx[s] - n + (r - cu_q[s]);
     }
-    const int g = h / (H / G);
-    const long qrow = (long)(row_base + r) * ldq + (long)h * dk;
-    for (int e = lane; e < dk; e += 64) qs[e] = ld1<B16>(q, qrow + e) * scale;
+    const int g = h0 / (H / G);
+    const long qrow = (long)(row_base + r) * ldq + (long)h0 * dk;
+    for (int e = lane; e < REP * dk; e += 64) qs[e] = ld1<B16>(q, qrow + e) * scale;
     int lo = chunk > 0 ? (pos / chunk) * chunk : window > 0 ? max(0, pos - window + 1) : 0;
     if (parts > 1) {  // this partition's keys; the sink joins in the merge
         lo += z * part_len;
@@ -93,27 +126,37 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
         sink = 0;
     }
     const int* table = bt + (long)s * bt_stride;
-    float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
-    float acc[DVU];
+    float m[REP], l[REP], acc[REP][DVU];
 #pragma unroll
-    for (int u = 0; u < DVU; ++u) acc[u] = 0.f;
+    for (int i = 0; i < REP; ++i) {
+        m[i] = sink ? 0.f : -INFINITY;
+        l[i] = sink ? 1.f : 0.f;
+#pragma unroll
+        for (int u = 0; u < DVU; ++u) acc[i][u] = 0.f;
+    }
     __syncthreads();
     for (int j0 = lo; j0 <= pos; j0 += 64) {
         const int j = j0 + lane;
         const bool ok = j <= pos;
-        float sc = -INFINITY;
+        float sc[REP];
         long tok = 0;
         if (ok) {
             tok = (long)table[j / bs] * bs + (j % bs);
-            sc = dot_row<B16>(kc, (tok * G + g) * dk, qs, dk);
+            dot_row<B16, REP>(kc, (tok * G + g) * dk, qs, dk, sc);
         }
-        const float mn = fmaxf(m, wave_max(sc));
-        const float p = ok ? expf(sc - mn) : 0.f;
-        const float alpha = expf(m - mn);  // 0 on the first tile without a sink (m = -inf, mn finite: the tile has key lo)
-        l = l * alpha + wave_sum(p);
-        m = mn;
+        float alpha[REP], p[REP];
+#pragma unroll
+        for (int i = 0; i < REP; ++i) {
+            const float si = ok ? sc[i] : -INFINITY;
+            const float mn = fmaxf(m[i], wave_max(si));
+            p[i] = ok ? expf(si - mn) : 0.f;
+            alpha[i] = expf(m[i] - mn);  // 0 on the first tile without a sink (m = -inf, mn finite: the tile has key lo)
+            l[i] = l[i] * alpha[i] + wave_sum(p[i]);
+            m[i] = mn;
+        }
         __syncthreads();  // the previous tile's weights and offsets have been read
-        ps[lane] = p;
+#pragma unroll
+        for (int i = 0; i < REP; ++i) ps[i * 64 + lane] = p[i];
         rowoff[lane] = (tok * G + g) * dv;
         __syncthreads();
         const int nk = min(64, pos - j0 + 1);
@@ -121,41 +164,54 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
         for (int u = 0; u < DVU; ++u) {
             const int c = lane + u * 64;
             if (c < dv) {
-                float a = acc[u] * alpha;
+                float a[REP];
+#pragma unroll
+                for (int i = 0; i < REP; ++i) a[i] = acc[i][u] * alpha[i];
                 int jj = 0;
-                for (; jj + 8 <= nk; jj += 8) {  // eight independent loads in flight, then their products
-                    float vv[8];
+                for (; jj + 16 <= nk; jj += 16) {  // sixteen independent loads in flight, then their products
+                    float vv[16];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) vv[e] = ld1<B16>(vc, rowoff[jj + e] + c);
+                    for (int e = 0; e < 16; ++e) vv[e] = ld1<B16>(vc, rowoff[jj + e] + c);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) a += ps[jj + e] * vv[e];
+                    for (int i = 0; i < REP; ++i)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) a[i] += ps[i * 64 + jj + e] * vv[e];
                 }
-                for (; jj < nk; ++jj) a += ps[jj] * ld1<B16>(vc, rowoff[jj] + c);
-                acc[u] = a;
+                for (; jj < nk; ++jj) {
+                    const float vv = ld1<B16>(vc, rowoff[jj] + c);
+#pragma unroll
+                    for (int i = 0; i < REP; ++i) a[i] += ps[i * 64 + jj] * vv;
+                }
+#pragma unroll
+                for (int i = 0; i < REP; ++i) acc[i][u] = a[i];
             }
         }
     }
-    if (parts > 1) {
-        const long pr = ((long)r * H + h) * parts + z;
-        if (lane == 0) {
-            part_ml[pr * 2] = m;
-            part_ml[pr * 2 + 1] = l;
+#pragma unroll
+    for (int i = 0; i < REP; ++i) {
+        const int h = h0 + i;
+        if (parts > 1) {
+            const long pr = ((long)r * H + h) * parts + z;
+            if (lane == 0) {
+                part_ml[pr * 2] = m[i];
+                part_ml[pr * 2 + 1] = l[i];
+            }
+#pragma unroll
+            for (int u = 0; u < DVU; ++u) {
+                const int c = lane + u * 64;
+                if (c < dv) part_o[pr * dv + c] = acc[i][u];
+            }
+            continue;
         }
+        const float inv = out_scale / l[i];
+        const long orow = (long)(row_base + r) * ldo + (long)h * dv;
 #pragma unroll
         for (int u = 0; u < DVU; ++u) {
             const int c = lane + u * 64;
-            if (c < dv) part_o[pr * dv + c] = acc[u];
-        }
-        return;
-    }
-    const float inv = out_scale / l;
-    const long orow = (long)(row_base + r) * ldo + (long)h * dv;
-#pragma unroll
-    for (int u = 0; u < DVU; ++u) {
-        const int c = lane + u * 64;
-        if (c < dv) {
-            if constexpr (O16) ((bf16_t*)out)[orow + c] = f32_to_bf16(acc[u] * inv);
-            else ((float*)out)[orow + c] = acc[u] * inv;
+            if (c < dv) {
+                if constexpr (O16) ((bf16_t*)out)[orow + c] = f32_to_bf16(acc[i][u] * inv);
+                else ((float*)out)[orow + c] = acc[i][u] * inv;
+            }
         }
     }
 }
@@ -171,6 +227,7 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* part_ml, co
     for (int z = 0; z < parts; ++z)
         if (part_ml[(p0 + z) * 2 + 1] > 0.f) M = fmaxf(M, part_ml[(p0 + z) * 2]);
     float L = sink ? expf(-M) : 0.f;
+    constexpr int DVU = DVU_MAX;
     float acc[DVU];
 #pragma unroll
     for (int u = 0; u < DVU; ++u) acc[u] = 0.f;
@@ -263,21 +320,31 @@ extern "C" int mxh_attention(const void* q, int ldq, int q16, const void* kc, co
                              float* part_ml, float* part_o, hipStream_t st) {
     if (n_rows <= 0 || n_seqs <= 0) return 0;
     MXH_CHECK(q && kc && vc && bt && ctx && out && bs > 0 && bt_stride > 0);
-    MXH_CHECK(H > 0 && G > 0 && H % G == 0 && dk > 0 && dv > 0 && dv <= 64 * DVU && dk <= 4096);
+    MXH_CHECK(H > 0 && G > 0 && H % G == 0 && dk > 0 && dv > 0 && dv <= 64 * DVU_MAX && dk <= 4096);
     MXH_CHECK(ldq >= H * dk && ldo >= H * dv && chunk >= 0 && window >= 0 && H <= 65535 && row_off >= 0);
     MXH_CHECK(cu_q || (row_off == 0 && n_rows == n_seqs));
     MXH_CHECK(parts >= 1 && parts <= 65535 && (parts == 1 || (!cu_q && part_len > 0 && part_ml && part_o)));
-    const dim3 grid(n_rows, H, parts);
-    const size_t sh = (size_t)(dk + 64 + 2) * sizeof(float) + 64 * sizeof(long);
-#define GO(B, O)                                                                                                    \
-    attn_rows_kernel<B, O><<<grid, 64, sh, st>>>(q, ldq, kc, vc, bs, bt, bt_stride, cu_q, ctx, n_seqs, row_base, out, \
-                                                 ldo, H, G, dk, dv, scale, chunk, window, sink, out_scale, row_off,  \
-                                                 parts, part_len, part_ml, part_o)
+    // REP query heads that share a key / value head could go to one wave (the kernel takes REP as a parameter), but a
+    // wave that serves four heads measured 3.7x slower than four waves that serve one each: the row kernel is bound by
+    // its dependent chains, not by the loads it would save. One head per wave.
+    constexpr int REP = 1;
+    const dim3 grid(n_rows, H / REP, parts);
+    const size_t sh = (size_t)(REP * dk + REP * 64 + 2) * sizeof(float) + 64 * sizeof(long);
+#define GO3(B, O, R, D)                                                                                               \
+    attn_rows_kernel<B, O, R, D><<<grid, 64, sh, st>>>(q, ldq, kc, vc, bs, bt, bt_stride, cu_q, ctx, n_seqs, row_base, \
+                                                       out, ldo, H, G, dk, dv, scale, chunk, window, sink, out_scale, \
+                                                       row_off, parts, part_len, part_ml, part_o)
+#define GO(B, O)                                  \
+    do {                                          \
+        if (dv <= 128) GO3(B, O, REP, 2);         \
+        else GO3(B, O, REP, DVU_MAX);             \
+    } while (0)
     if (q16 && o16) GO(true, true);
     else if (q16) GO(true, false);
     else if (o16) GO(false, true);
     else GO(false, false);
 #undef GO
+#undef GO3
     if (parts > 1) {
         const dim3 g2(n_rows, H);
         if (o16) attn_merge_kernel<true><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, row_base, out, ldo);

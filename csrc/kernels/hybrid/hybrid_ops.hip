@@ -232,12 +232,13 @@ __global__ __launch_bounds__(NT) void conv_tails_kernel(const float* x, int ldx,
     }
 }
 
-// grid (T, heads), one wave per head
-__global__ __launch_bounds__(64) void unit_norm_kernel(float* x, int ldx, int dim, float eps, float scale) {
+// grid (T, heads), one wave per head; heads from `split` on take scale2
+__global__ __launch_bounds__(64) void unit_norm_kernel(float* x, int ldx, int dim, float eps, float scale, int split,
+                                                       float scale2) {
     float* p = x + (long)blockIdx.x * ldx + (long)blockIdx.y * dim;
     float ss = 0.f;
     for (int e = threadIdx.x; e < dim; e += 64) ss += p[e] * p[e];
-    const float sc = scale / sqrtf(wave_sum(ss) + eps);
+    const float sc = ((int)blockIdx.y < split ? scale : scale2) / sqrtf(wave_sum(ss) + eps);
     for (int e = threadIdx.x; e < dim; e += 64) p[e] *= sc;
 }
 
@@ -423,10 +424,11 @@ extern "C" int mxh_causal_conv(const float* x, int ldx, const float* w, const fl
     return (int)hipGetLastError();
 }
 
-extern "C" int mxh_unit_norm(float* x, int ldx, int heads, int dim, float eps, float scale, int T, hipStream_t st) {
+extern "C" int mxh_unit_norm(float* x, int ldx, int heads, int dim, float eps, float scale, int split, float scale2,
+                             int T, hipStream_t st) {
     if (T <= 0) return 0;
-    MXH_CHECK(x && heads > 0 && dim > 0 && ldx >= heads * dim);
-    unit_norm_kernel<<<dim3(T, heads), 64, 0, st>>>(x, ldx, dim, eps, scale);
+    MXH_CHECK(x && heads > 0 && heads <= 65535 && dim > 0 && ldx >= heads * dim);
+    unit_norm_kernel<<<dim3(T, heads), 64, 0, st>>>(x, ldx, dim, eps, scale, split, scale2);
     return (int)hipGetLastError();
 }
 

@@ -160,8 +160,8 @@ HYBRID_SIGS = {
     "mxh_masked_softmax": [P, P, I, L, I, I, I, I, F, I, I, I, P],
     # x, ldx, w, bias, taps, silu, tails, state, positions, n_dec, pf_cu, n_pf, out, ldo, T, C, stream
     "mxh_causal_conv": [P, I, P, P, I, I, P, P, P, I, P, I, P, I, I, I, P],
-    # x, ldx, heads, dim, eps, scale, T, stream
-    "mxh_unit_norm": [P, I, I, I, F, F, I, P],
+    # x, ldx, heads, dim, eps, scale, split, scale2, T, stream
+    "mxh_unit_norm": [P, I, I, I, F, F, I, F, I, P],
     # a, lda, b, ldb, A_log, dt_bias, decay, coef, T, H, stream
     "mxh_scan_coefs": [P, I, P, I, P, P, P, P, I, I, P],
     # k, ldk, q, ldq, v, ldv, decay, coef, skip, state, seq_state, positions, n_dec, pf_cu, n_pf, out, ldo, H, G, N, P,

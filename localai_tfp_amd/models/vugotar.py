@@ -552,8 +552,7 @@ class VugotarModel:
         cc = 2 * nq + nv
         xc = ws.conv[:T * cc].view(T, cc)
         HY.causal_conv(y[:, c["rq"]:c["rq"] + cc], W.conv_w, None, tails, rag, xc, silu=True)
-        HY.unit_norm_heads(xc[:, :nq], G, dk, DELTA_UNIT_EPS, dk ** -0.5)
-        HY.unit_norm_heads(xc[:, nq:2 * nq], G, dk, DELTA_UNIT_EPS, 1.0)
+        HY.unit_norm_heads(xc[:, :2 * nq], 2 * G, dk, DELTA_UNIT_EPS, dk ** -0.5, split=G, scale2=1.0)  # q | k
         decay, coef = ws.decay[:T * H].view(T, H), ws.coef[:T * H].view(T, H)
         HY.scan_coefs(y[:, c["ra"]:c["ra"] + H], y[:, c["rb"]:c["rb"] + H], W.A_log, W.dt_bias, decay, coef)
         o = ws.scan[:T * nv].view(T, nv)

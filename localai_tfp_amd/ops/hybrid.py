@@ -148,10 +148,10 @@ DECODE_WAVES = 4096  # decode rows: waves to aim for when splitting contexts int
 
 def decode_part_len(n_dec: int, heads: int, visible: int) -> int:
     """Keys per partition of the decode rows: one wave walks a (row, head, partition), so few sequences with long
-    visible ranges are split finely (down to two 64-key tiles) and large batches coarsely."""
+    visible ranges are split finely (down to one 64-key tile) and large batches coarsely."""
     want = max(1, DECODE_WAVES // max(1, n_dec * heads))
     per = -(-max(1, visible) // want)
-    return max(128, -(-per // 64) * 64)
+    return max(64, -(-per // 64) * 64)
 
 
 def _visible_blocks(p0: int, n: int, chunk: int, window: int, heads: int):
@@ -321,17 +321,23 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, tai
 
 
 # ------------------------------------------------------------------------------------------------ recurrences
-def unit_norm_heads(x: torch.Tensor, heads: int, dim: int, eps: float, scale: float = 1.0):
-    """In place on fp32 x [T, heads*dim]: every head becomes x / sqrt(sum(x^2) + eps) * scale."""
+def unit_norm_heads(x: torch.Tensor, heads: int, dim: int, eps: float, scale: float = 1.0, split: int | None = None,
+                    scale2: float = 1.0):
+    """In place on fp32 x [T, heads*dim]: every head becomes x / sqrt(sum(x^2) + eps) * scale; heads from index
+    `split` on are multiplied by scale2 instead (queries and keys that lie side by side in one launch)."""
     T = x.shape[0]
     if T == 0:
         return x
+    split = heads if split is None else split
     if not x.is_cuda:
         v = x.reshape(T, heads, dim)
-        x.copy_((v * torch.rsqrt(v.pow(2).sum(-1, keepdim=True) + eps) * scale).reshape(T, heads * dim))
+        sc = torch.full((heads, 1), float(scale))
+        sc[split:] = scale2
+        x.copy_((v * torch.rsqrt(v.pow(2).sum(-1, keepdim=True) + eps) * sc).reshape(T, heads * dim))
         return x
     _f32c(x, "unit_norm_heads")
-    N.kcall("mxh_unit_norm", x.data_ptr(), x.stride(0), heads, dim, float(eps), float(scale), T, N.stream_ptr())
+    N.kcall("mxh_unit_norm", x.data_ptr(), x.stride(0), heads, dim, float(eps), float(scale), int(split), float(scale2),
+            T, N.stream_ptr())
     return x
 
 
