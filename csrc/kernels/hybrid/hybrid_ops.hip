@@ -31,7 +31,6 @@ MX_DEV float block_sum_dyn(float v, float* red) {
     v = wave_sum(v);
     const int nw = blockDim.x >> 6;
     if (nw == 1) return v;
-    __syncthreads();
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
     __syncthreads();
     float s = 0.f;
@@ -62,13 +61,14 @@ __global__ __launch_bounds__(NT) void offset_norm_kernel(const float* x, int ldx
     const int i = blockIdx.x;
     const float* xr = x + (long)(rows ? rows[i] : i) * ldx;
     const bool cached = C <= NT * RC;
-    float keep[RC];
+    float keep[RC], wk[RC];
     float ss = 0.f;
     if (cached) {
 #pragma unroll
         for (int k = 0; k < RC; ++k) {  // clamped addresses: straight-line loads, all in flight together
             const int c = threadIdx.x + k * NT;
             const float v = xr[min(c, C - 1)];
+            wk[k] = w[min(c, C - 1)];  // requested with the row, not after the reduction
             keep[k] = c < C ? v : 0.f;
             ss += keep[k] * keep[k];
         }
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(NT) void offset_norm_kernel(const float* x, int ldx
         for (int k = 0; k < RC; ++k) {
             const int c = threadIdx.x + k * NT;
             if (c < C) {
-                const float v = keep[k] * sc * (offset + w[c]);
+                const float v = keep[k] * sc * (offset + wk[k]);
                 if (o32) o32[(long)i * ld32 + c] = v;
                 if (o16) o16[(long)i * ld16 + c] = f32_to_bf16(v);
             }
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(64) void rope_norm_append_kernel(const float* qi, c
 
 // grid (ceil(C / NT), sequences, ceil(T / CONV_ROWS)): thread = channel. Reads the tails only; conv_tails_kernel
 // rolls them afterwards
-constexpr int CONV_ROWS = 32;
+constexpr int CONV_ROWS = 8;
 __global__ __launch_bounds__(NT) void causal_conv_kernel(const float* x, int ldx, const float* w, const float* bias,
                                                          int taps, int silu, float* tails, const int* state,
                                                          const int* positions, int n_dec, const int* pf_cu, float* out,
@@ -253,7 +253,9 @@ __global__ __launch_bounds__(NT) void scan_coefs_kernel(const float* a, int lda,
     coef[i] = b ? sigmoid_acc(b[(long)t * ldb + h]) : s;
 }
 
-// grid (T, C / group): one block per (token, group of columns)
+// grid (T, C / group): one block per (token, group of columns). Groups of up to blockDim * GC numbers are read once
+// (straight-line clamped loads, all in flight together) and kept in registers with their gates
+constexpr int GC = 32;
 template <bool B16>
 __global__ void gated_group_norm_kernel(const float* y, int ldy, const float* gate, int ldg, const float* w, int wlen,
                                         float eps, int group, int gate_first, float out_scale, void* out, int ldo) {
@@ -261,15 +263,43 @@ __global__ void gated_group_norm_kernel(const float* y, int ldy, const float* ga
     const int t = blockIdx.x, c0 = blockIdx.y * group;
     const float* yr = y + (long)t * ldy + c0;
     const float* gr = gate + (long)t * ldg + c0;
+    const int nt = blockDim.x;
+    if (group <= nt * GC) {
+        float z[GC], gs[GC];
+        float ss = 0.f;
+#pragma unroll
+        for (int k = 0; k < GC; ++k) {
+            const int e = threadIdx.x + k * nt;
+            if (k * nt < group) {  // uniform: whole rounds beyond the group are skipped
+                const int ec = min(e, group - 1);
+                const float yv = yr[ec], gv = gr[ec];
+                gs[k] = silu_acc(gv);
+                z[k] = e < group ? (gate_first ? yv * gs[k] : yv) : 0.f;
+                ss += z[k] * z[k];
+            }
+        }
+        ss = block_sum_dyn(ss, red);
+        const float sc = out_scale / sqrtf(ss / (float)group + eps);
+#pragma unroll
+        for (int k = 0; k < GC; ++k) {
+            const int e = threadIdx.x + k * nt;
+            if (k * nt < group && e < group) {
+                float v = z[k] * sc * w[(c0 + e) % wlen];
+                if (!gate_first) v *= gs[k];
+                st_elem<B16>(out, (long)t * ldo + c0 + e, v);
+            }
+        }
+        return;
+    }
     float ss = 0.f;
-    for (int e = threadIdx.x; e < group; e += blockDim.x) {
+    for (int e = threadIdx.x; e < group; e += nt) {
         float v = yr[e];
         if (gate_first) v *= silu_acc(gr[e]);
         ss += v * v;
     }
     ss = block_sum_dyn(ss, red);
     const float sc = out_scale / sqrtf(ss / (float)group + eps);
-    for (int e = threadIdx.x; e < group; e += blockDim.x) {
+    for (int e = threadIdx.x; e < group; e += nt) {
         const float g = silu_acc(gr[e]);
         float v = yr[e];
         if (gate_first) v *= g;

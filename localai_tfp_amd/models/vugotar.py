@@ -326,7 +326,7 @@ class VugotarWorkspace:
         # partial results of decode rows whose visible keys are split into partitions
         h_att = max([L.mixer.left.heads for L in cfg.layers if L.type == "parallel"] or [1])
         v_att = max([L.mixer.left.vdim for L in cfg.layers if L.type == "parallel"] or [1])
-        rows = max_seqs * h_att * max(1, min(max_parts, 64))
+        rows = HY.DECODE_WAVES + max_seqs * h_att  # few sequences take many partitions each, many take few
         self.part_ml = torch.empty((rows, 2), **f32)
         self.part_o = torch.empty((rows, v_att), **f32)
 

@@ -327,6 +327,10 @@ def test_unit_heads_group_norm_glu_and_router(dev):
     v = x[:, 3:].double().reshape(T, 4, 10)
     close(xd[:, 3:], (v / torch.sqrt((v * v).sum(-1, keepdim=True) + 1e-6) * 10 ** -0.5).reshape(T, 40), 1e-5)
     assert torch.equal(xd[:, :3].cpu(), x[:, :3])
+    xd = x.clone().to(dev)  # queries and keys side by side: the first three heads scaled, the last one not
+    HY.unit_norm_heads(xd[:, 3:], 4, 10, 1e-6, 0.25, split=3, scale2=1.0)
+    sc = torch.tensor([0.25, 0.25, 0.25, 1.0], dtype=torch.float64)[None, :, None]
+    close(xd[:, 3:], (v / torch.sqrt((v * v).sum(-1, keepdim=True) + 1e-6) * sc).reshape(T, 40), 1e-5)
     # group norm: gate before the norm over 3 groups with a full-width weight; gate after it with a per-head weight
     y, gt = torch.randn(T, 36, generator=g), torch.randn(T, 36 + 2, generator=g)
     w_full, w_head = torch.randn(36, generator=g), torch.randn(12, generator=g)
