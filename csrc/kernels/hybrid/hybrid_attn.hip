@@ -216,40 +216,40 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
     }
 }
 
-// grid (rows, H): combines the partitions of a row in order; an empty partition has sum 0
+// grid (rows, H): combines the partitions of a row (at most 64: lane z holds partition z's maximum and sum) in a fixed
+// order; an empty partition has sum 0
 template <bool O16>
 __global__ __launch_bounds__(64) void attn_merge_kernel(const float* part_ml, const float* part_o, int parts, int H,
                                                         int dv, int sink, float out_scale, int row_base, void* out,
                                                         int ldo) {
+    constexpr int DVU = DVU_MAX;
     const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const long p0 = ((long)r * H + h) * parts;
-    float M = sink ? 0.f : -INFINITY;
-    for (int z = 0; z < parts; ++z)
-        if (part_ml[(p0 + z) * 2 + 1] > 0.f) M = fmaxf(M, part_ml[(p0 + z) * 2]);
-    float L = sink ? expf(-M) : 0.f;
-    constexpr int DVU = DVU_MAX;
-    float acc[DVU];
-#pragma unroll
-    for (int u = 0; u < DVU; ++u) acc[u] = 0.f;
-    for (int z = 0; z < parts; ++z) {
-        const float lz = part_ml[(p0 + z) * 2 + 1];
-        if (!(lz > 0.f)) continue;
-        const float w = expf(part_ml[(p0 + z) * 2] - M);
-        L += lz * w;
-#pragma unroll
-        for (int u = 0; u < DVU; ++u) {
-            const int c = lane + u * 64;
-            if (c < dv) acc[u] += part_o[(p0 + z) * dv + c] * w;
-        }
-    }
+    const int zc = min(lane, parts - 1);
+    const float mz = part_ml[(p0 + zc) * 2], lz = lane < parts ? part_ml[(p0 + zc) * 2 + 1] : 0.f;
+    float M = wave_max(lz > 0.f ? mz : -INFINITY);
+    if (sink) M = fmaxf(M, 0.f);
+    const float w = lz > 0.f ? expf(mz - M) : 0.f;
+    const float L = wave_sum(lz * w) + (sink ? expf(-M) : 0.f);
     const float inv = out_scale / L;
     const long orow = (long)(row_base + r) * ldo + (long)h * dv;
 #pragma unroll
     for (int u = 0; u < DVU; ++u) {
         const int c = lane + u * 64;
-        if (c < dv) {
-            if constexpr (O16) ((bf16_t*)out)[orow + c] = f32_to_bf16(acc[u] * inv);
-            else ((float*)out)[orow + c] = acc[u] * inv;
+        if (u * 64 < dv) {
+            const int cc = min(c, dv - 1);
+            float a = 0.f;
+            for (int z0 = 0; z0 < parts; z0 += 8) {  // eight partitions' numbers requested together
+                float x[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = part_o[(p0 + min(z0 + e, parts - 1)) * dv + cc];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a += x[e] * __shfl(w, min(z0 + e, 63), 64) * (z0 + e < parts ? 1.f : 0.f);
+            }
+            if (c < dv) {
+                if constexpr (O16) ((bf16_t*)out)[orow + c] = f32_to_bf16(a * inv);
+                else ((float*)out)[orow + c] = a * inv;
+            }
         }
     }
 }
@@ -323,7 +323,7 @@ extern "C" int mxh_attention(const void* q, int ldq, int q16, const void* kc, co
     MXH_CHECK(H > 0 && G > 0 && H % G == 0 && dk > 0 && dv > 0 && dv <= 64 * DVU_MAX && dk <= 4096);
     MXH_CHECK(ldq >= H * dk && ldo >= H * dv && chunk >= 0 && window >= 0 && H <= 65535 && row_off >= 0);
     MXH_CHECK(cu_q || (row_off == 0 && n_rows == n_seqs));
-    MXH_CHECK(parts >= 1 && parts <= 65535 && (parts == 1 || (!cu_q && part_len > 0 && part_ml && part_o)));
+    MXH_CHECK(parts >= 1 && parts <= 64 && (parts == 1 || (!cu_q && part_len > 0 && part_ml && part_o)));
     // REP query heads that share a key / value head could go to one wave (the kernel takes REP as a parameter), but a
     // wave that serves four heads measured 3.7x slower than four waves that serve one each: the row kernel is bound by
     // its dependent chains, not by the loads it would save. One head per wave.

@@ -268,15 +268,17 @@ __global__ void gated_group_norm_kernel(const float* y, int ldy, const float* ga
         float z[GC], gs[GC];
         float ss = 0.f;
 #pragma unroll
+        for (int k = 0; k < GC; ++k) {  // no branch in this loop: the loads are requested back to back
+            const int ec = min((int)threadIdx.x + k * nt, group - 1);
+            z[k] = yr[ec];
+            gs[k] = gr[ec];
+        }
+#pragma unroll
         for (int k = 0; k < GC; ++k) {
             const int e = threadIdx.x + k * nt;
-            if (k * nt < group) {  // uniform: whole rounds beyond the group are skipped
-                const int ec = min(e, group - 1);
-                const float yv = yr[ec], gv = gr[ec];
-                gs[k] = silu_acc(gv);
-                z[k] = e < group ? (gate_first ? yv * gs[k] : yv) : 0.f;
-                ss += z[k] * z[k];
-            }
+            gs[k] = silu_acc(gs[k]);
+            z[k] = e < group ? (gate_first ? z[k] * gs[k] : z[k]) : 0.f;
+            ss += z[k] * z[k];
         }
         ss = block_sum_dyn(ss, red);
         const float sc = out_scale / sqrtf(ss / (float)group + eps);

@@ -246,7 +246,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
         if workspace is not None:
             plen = decode_part_len(nd, H, vis)
             parts = -(-vis // plen)
-            room = workspace[0].shape[0] // (nd * H)
+            room = min(64, workspace[0].shape[0] // (nd * H))  # the merge holds one partition per lane
             if parts > room:
                 parts = max(1, room)
                 plen = -(-(-(-vis // parts)) // 64) * 64
