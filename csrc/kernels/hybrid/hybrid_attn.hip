@@ -34,8 +34,8 @@ MX_DEV float dot8(const uint4 w, const float* qq) {
 MX_DEV float dot4(const float4 w, const float* qq) { return w.x * qq[0] + w.y * qq[1] + w.z * qq[2] + w.w * qq[3]; }
 
 // dots of one pool row with REP fp32 queries in LDS (q + r * n; n numbers, row and queries 16-byte aligned when
-// n % 8 == 0). Four 16-byte pieces of the row are requested before the first is used: a lane's loads are one
-// dependent chain otherwise. The row is read once for all REP queries.
+// n % 8 == 0). Eight (fp32: four) 16-byte pieces of the row are requested before the first is used: a lane's loads
+// are one dependent chain otherwise. The row is read once for all REP queries.
 template <bool B16, int REP>
 MX_DEV void dot_row(const void* base, long off, const float* q, int n, float (&acc)[REP]) {
 #pragma unroll
@@ -45,6 +45,17 @@ MX_DEV void dot_row(const void* base, long off, const float* q, int n, float (&a
             const uint4* p = (const uint4*)((const bf16_t*)base + off);
             const int m = n / 8;
             int i = 0;
+            for (; i + 8 <= m; i += 8) {
+                uint4 w[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) w[e] = p[i + e];
+#pragma unroll
+                for (int r = 0; r < REP; ++r) {
+                    const float* qq = q + r * n + i * 8;
+                    acc[r] += ((dot8(w[0], qq) + dot8(w[1], qq + 8)) + (dot8(w[2], qq + 16) + dot8(w[3], qq + 24))) +
+                              ((dot8(w[4], qq + 32) + dot8(w[5], qq + 40)) + (dot8(w[6], qq + 48) + dot8(w[7], qq + 56)));
+                }
+            }
             for (; i + 4 <= m; i += 4) {
                 const uint4 w0 = p[i], w1 = p[i + 1], w2 = p[i + 2], w3 = p[i + 3];
 #pragma unroll
@@ -160,30 +171,33 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
         rowoff[lane] = (tok * G + g) * dv;
         __syncthreads();
         const int nk = min(64, pos - j0 + 1);
+        // VB keys' values for all of the lane's columns are requested together (clamped columns: no branch between
+        // the loads), then multiplied in
+        constexpr int VB = DVU <= 2 ? 16 : 4;
 #pragma unroll
-        for (int u = 0; u < DVU; ++u) {
-            const int c = lane + u * 64;
-            if (c < dv) {
-                float a[REP];
+        for (int i = 0; i < REP; ++i)
 #pragma unroll
-                for (int i = 0; i < REP; ++i) a[i] = acc[i][u] * alpha[i];
-                int jj = 0;
-                for (; jj + 16 <= nk; jj += 16) {  // sixteen independent loads in flight, then their products
-                    float vv[16];
+            for (int u = 0; u < DVU; ++u) acc[i][u] *= alpha[i];
+        int jj = 0;
+        for (; jj + VB <= nk; jj += VB) {
+            float vv[DVU][VB];
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) vv[e] = ld1<B16>(vc, rowoff[jj + e] + c);
+            for (int u = 0; u < DVU; ++u)
 #pragma unroll
-                    for (int i = 0; i < REP; ++i)
+                for (int e = 0; e < VB; ++e) vv[u][e] = ld1<B16>(vc, rowoff[jj + e] + min(lane + u * 64, dv - 1));
 #pragma unroll
-                        for (int e = 0; e < 16; ++e) a[i] += ps[i * 64 + jj + e] * vv[e];
-                }
-                for (; jj < nk; ++jj) {
-                    const float vv = ld1<B16>(vc, rowoff[jj] + c);
+            for (int i = 0; i < REP; ++i)
 #pragma unroll
-                    for (int i = 0; i < REP; ++i) a[i] += ps[i * 64 + jj] * vv;
-                }
+                for (int u = 0; u < DVU; ++u)
 #pragma unroll
-                for (int i = 0; i < REP; ++i) acc[i][u] = a[i];
+                    for (int e = 0; e < VB; ++e) acc[i][u] += ps[i * 64 + jj + e] * vv[u][e];
+        }
+        for (; jj < nk; ++jj) {
+#pragma unroll
+            for (int u = 0; u < DVU; ++u) {
+                const float vv = ld1<B16>(vc, rowoff[jj] + min(lane + u * 64, dv - 1));
+#pragma unroll
+                for (int i = 0; i < REP; ++i) acc[i][u] += ps[i * 64 + jj] * vv;
             }
         }
     }
