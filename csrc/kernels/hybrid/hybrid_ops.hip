@@ -254,9 +254,9 @@ __global__ __launch_bounds__(NT) void scan_coefs_kernel(const float* a, int lda,
 }
 
 // grid (T, C / group): one block per (token, group of columns). Groups of up to blockDim * GC numbers are read once
-// (straight-line clamped loads, all in flight together) and kept in registers with their gates
-constexpr int GC = 32;
-template <bool B16>
+// (straight-line clamped loads, all in flight together) and kept in registers with their gates; the launcher picks
+// the smallest GC that holds the group
+template <bool B16, int GC>
 __global__ void gated_group_norm_kernel(const float* y, int ldy, const float* gate, int ldg, const float* w, int wlen,
                                         float eps, int group, int gate_first, float out_scale, void* out, int ldo) {
     __shared__ float red[NT / 64];
@@ -479,11 +479,18 @@ extern "C" int mxh_gated_group_norm(const float* y, int ldy, const float* gate, 
     MXH_CHECK(y && gate && w && out && C > 0 && group > 0 && C % group == 0 && wlen > 0 && C % wlen == 0);
     MXH_CHECK(ldy >= C && ldg >= C && ldo >= C);
     const dim3 grid(T, C / group);
-    const int nt = group <= 256 ? 64 : NT;
-    if (o16) gated_group_norm_kernel<true><<<grid, nt, 0, st>>>(y, ldy, gate, ldg, w, wlen, eps, group, gate_first,
-                                                                out_scale, out, ldo);
-    else gated_group_norm_kernel<false><<<grid, nt, 0, st>>>(y, ldy, gate, ldg, w, wlen, eps, group, gate_first,
-                                                             out_scale, out, ldo);
+#define GO(B, G_, nt_) \
+    gated_group_norm_kernel<B, G_><<<grid, nt_, 0, st>>>(y, ldy, gate, ldg, w, wlen, eps, group, gate_first, out_scale, out, ldo)
+#define PICK(B)                              \
+    do {                                     \
+        if (group <= 256) GO(B, 4, 64);      \
+        else if (group <= 2048) GO(B, 8, NT); \
+        else GO(B, 32, NT);                  \
+    } while (0)
+    if (o16) PICK(true);
+    else PICK(false);
+#undef PICK
+#undef GO
     return (int)hipGetLastError();
 }
 
