@@ -319,7 +319,7 @@ class VugotarWorkspace:
         self.coef = torch.empty((T * n_heads,), **f32)
         self.scan = torch.empty((T * n_scan,), **f32)
         self.q = torch.empty((T * n_q,), **m16)
-        self.cat = torch.empty((T * k_out,), **m16)
+        self.cat = torch.zeros((T * k_out,), **m16)  # zero: padded columns are read, never written
         self.route = torch.empty((T * n_e,), **f32)
         self.hs = torch.empty((S, C), **m16)
         self.logits = torch.empty((S, cfg.vocab), **f32)
@@ -460,9 +460,16 @@ class VugotarModel:
                 add("egate", torch.cat([t(f"{q}e{e}.gate", (f.ff, C)) for e in range(f.experts)], 0))
                 add("eup", torch.cat([t(f"{q}e{e}.up", (f.ff, C)) for e in range(f.experts)], 0))
                 outs += [t(f"{q}e{e}.down", (C, f.ff)) for e in range(f.experts)]
-            w_out = torch.cat(outs, 1)
+            # both stacked GEMMs get whole 16-byte rows: zero rows / columns up to a multiple of 8 (the padded columns
+            # of the output GEMM's operand are never written and stay zero)
+            w_in, w_out = torch.cat(rows, 0), torch.cat(outs, 1)
+            if n % 8:
+                w_in = torch.cat([w_in, torch.zeros(8 - n % 8, C)], 0)
+                n = w_in.shape[0]
+            if w_out.shape[1] % 8:
+                w_out = torch.cat([w_out, torch.zeros(C, 8 - w_out.shape[1] % 8)], 1)
             m.weights[i] = VugotarWeights(
-                norm=f32(f"l{i}.norm1", (C,)), w_in=Dense(torch.cat(rows, 0), None, dev, md),
+                norm=f32(f"l{i}.norm1", (C,)), w_in=Dense(w_in, None, dev, md),
                 w_out=Dense(w_out, out_b, dev, md), cols=cols, n_in=n, k_out=w_out.shape[1],
                 conv_w=conv_w.contiguous().to(dev), conv_b=conv_b, A_log=A_log, dt_bias=dt_bias, mix_norm=mix_norm,
                 skip=skip, gate_b=gate_b, up_b=up_b)

@@ -262,8 +262,8 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
             N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
                     rag.pf_bt.data_ptr(), rag.pf_bt.stride(0), rag.pf_cu.data_ptr(), rag.pf_ctx.data_ptr(), rag.n_pf,
                     n_rows, nd, out.data_ptr(), out.stride(0), _is16(out), *common, row_off, 1, 0, None, None, st)
-        if lens is None or max(lens) < GEMM_MIN_ROWS:
-            rows_kernel(0, T - nd)
+        if lens is None or max(lens) < GEMM_MIN_ROWS or 0 < chunk < GEMM_MIN_ROWS:
+            rows_kernel(0, T - nd)  # (chunks shorter than a block of rows: a row's few visible keys suit the row kernel)
             return out
         r, run0 = 0, None  # run0: first row of a run of consecutive short chunks
         for k, n in enumerate(lens):

@@ -34,11 +34,11 @@ SHAPES = {
                   router_scale=1.5, left_scale=0.6, right_scale=0.9, loop=(0, 2, 2)),
     # sizes that differ from each other: dim != vdim, partial rotation, a chunk smaller than a page and odd, as many
     # key heads as heads, two taps and five taps, a state size that is no power of two, top == experts, no shared
-    # expert, a layer without a feed-forward, no loop, a large eps
+    # expert, a layer without a feed-forward, no loop, a large eps, stacked projections of odd total width
     "odd": dict(hidden=40, vocab=61, pattern=("mamba2", "parallel", "parallel"), mlps=(None, "moe", "dense"), heads=6,
                 kv_heads=3, dim=24, vdim=40, chunk=7, rot_dims=8, rot_base=300.0, scale=0.4, d_heads=3, d_kv_heads=3,
                 d_dim=20, d_vdim=12, d_conv=2, m_heads=3, m_vdim=24, m_state=40, m_groups=3, m_norm_groups=1, m_conv=5,
-                ff=50, experts=5, top=5, expert_ff=18, shared_ff=0, router_scale=0.7, left_scale=1.4, right_scale=0.5,
+                ff=50, experts=5, top=5, expert_ff=17, shared_ff=0, router_scale=0.7, left_scale=1.4, right_scale=0.5,
                 eps=1e-3),
     # states wider than a lane keeps alone (96 and 160 numbers per column), value sizes that are no multiple of 64,
     # one expert of many, one key head for all heads, the loop over the last layer only
