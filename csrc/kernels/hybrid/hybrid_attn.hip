@@ -230,6 +230,184 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
     }
 }
 
+// attn_chunk_mfma_kernel: a prompt chunk of one sequence on the matrix cores (bf16 pools, head sizes that are
+// multiples of 32 / 16). A workgroup of 4 waves owns RT 16-row query tiles of GW query heads that share a key / value
+// head (GW * RT = 4); a wave owns one tile of one head, its query fragments in registers. Keys are taken 64 at a time:
+// the workgroup stages the key tile [64][DK] and the transposed value tile [DV][64] in LDS (the next tile's numbers are
+// requested from memory before the current tile is worked on and wait in registers), each wave forms S = Q K^T with
+// MFMA 16x16x32, masks (causal, chunk or window start) and updates its rows' running maximum and sum in fp32 (the sink
+// starts them at 0 and 1), writes the weights as bf16 to its own LDS patch and accumulates O += P V.
+// Fragment layout of v_mfma_f32_16x16x32_bf16 (g = lane / 16, col = lane % 16): A holds row col, k = 8g .. 8g + 7;
+// B holds column col, k = 8g .. 8g + 7; the result holds rows 4g .. 4g + 3 of column col.
+template <int DK, int DV, bool O16>
+__global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __restrict__ q, int ldq,
+                                                              const bf16_t* __restrict__ kc,
+                                                              const bf16_t* __restrict__ vc, int bs,
+                                                              const int* __restrict__ table, int p0, int n, void* out,
+                                                              int ldo, int H, int G, int GW, float scale, int chunk,
+                                                              int window, int sink, float out_scale) {
+    constexpr int KT = 64;
+    constexpr int KSTR = (DK + 8) * 2;  // bytes per key row in LDS (padded)
+    constexpr int VSTR = (KT + 8) * 2;  // bytes per transposed value row (one dim, 64 keys)
+    constexpr int PSTR = (KT + 8) * 2;  // bytes per weight row
+    constexpr float LOG2E_ = 1.4426950408889634f;
+    __shared__ __attribute__((aligned(16))) char k_lds[KT * KSTR];
+    __shared__ __attribute__((aligned(16))) char v_lds[DV * VSTR];
+    __shared__ __attribute__((aligned(16))) char p_lds[4 * 16 * PSTR];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int g = lane >> 4, col = lane & 15;
+    const int RT = 4 / GW;
+    const int hq = blockIdx.y * GW + (wave % GW);
+    const int kvh = (blockIdx.y * GW) / (H / G);
+    // the chunk's last rows see the most keys: their workgroups are scheduled first
+    const int q0 = (gridDim.x - 1 - blockIdx.x) * RT * 16;  // first query row of the workgroup
+    const int row_q0 = q0 + (wave / GW) * 16;     // first query row of this wave
+    const int a_pos = p0 + q0;                    // position of the workgroup's first row
+    const int kv_end = p0 + min(n, q0 + RT * 16);  // one past the last visible key
+    const int kt_begin = chunk > 0 ? (a_pos / chunk) * chunk : window > 0 ? max(0, a_pos - window + 1) : 0;
+    const float qs = scale * LOG2E_;
+
+    bf16x8 qf[DK / 32];
+    {
+        const int qi = row_q0 + col;
+#pragma unroll
+        for (int ks = 0; ks < DK / 32; ++ks) {
+            if (qi < n) qf[ks] = *(const bf16x8*)(q + (size_t)qi * ldq + (size_t)hq * DK + 32 * ks + 8 * g);
+            else qf[ks] = (bf16x8){};
+        }
+    }
+    f32x4 oacc[DV / 16];
+#pragma unroll
+    for (int i = 0; i < DV / 16; ++i) oacc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float mrow[4], lrow[4];
+    int lo_row[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        mrow[i] = sink ? 0.f : -INFINITY;
+        lrow[i] = sink ? 1.f : 0.f;
+        const int qpos = p0 + row_q0 + 4 * g + i;
+        lo_row[i] = chunk > 0 ? (qpos / chunk) * chunk : window > 0 ? max(0, qpos - window + 1) : 0;
+    }
+    char* pw = p_lds + wave * 16 * PSTR;
+
+    constexpr int KCH = KT * DK / 8 / 256, VCH = KT * DV / 8 / 256;  // 16-byte pieces per thread
+    uint4 kr[KCH], vr[VCH];
+    auto load_tile = [&](int kt0) {
+#pragma unroll
+        for (int j = 0; j < KCH; ++j) {
+            const int id = threadIdx.x + j * 256;
+            const int p = id / (DK / 8), c = id % (DK / 8);
+            const int pos = min(kt0 + p, kv_end - 1);  // clamped: keys past the end are masked below
+            const size_t tok = (size_t)table[pos / bs] * bs + (pos % bs);
+            kr[j] = *(const uint4*)(kc + (tok * G + kvh) * DK + c * 8);
+        }
+#pragma unroll
+        for (int j = 0; j < VCH; ++j) {
+            const int id = threadIdx.x + j * 256;
+            const int p = id / (DV / 8), c = id % (DV / 8);
+            const int pos = min(kt0 + p, kv_end - 1);
+            const size_t tok = (size_t)table[pos / bs] * bs + (pos % bs);
+            vr[j] = *(const uint4*)(vc + (tok * G + kvh) * DV + c * 8);
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int j = 0; j < KCH; ++j) {
+            const int id = threadIdx.x + j * 256;
+            const int p = id / (DK / 8), c = id % (DK / 8);
+            *(uint4*)(k_lds + p * KSTR + c * 16) = kr[j];
+        }
+#pragma unroll
+        for (int j = 0; j < VCH; ++j) {
+            const int id = threadIdx.x + j * 256;
+            const int p = id / (DV / 8), c = id % (DV / 8);
+            const uint32_t w[4] = {vr[j].x, vr[j].y, vr[j].z, vr[j].w};
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj)
+                *(bf16_t*)(v_lds + (8 * c + jj) * VSTR + 2 * p) = (bf16_t)(w[jj >> 1] >> (16 * (jj & 1)));
+        }
+    };
+    if (kt_begin < kv_end) load_tile(kt_begin);
+    for (int kt0 = kt_begin; kt0 < kv_end; kt0 += KT) {
+        store_tile();
+        if (kt0 + KT < kv_end) load_tile(kt0 + KT);
+        __syncthreads();
+        // ---- S = Q K^T : 16 rows x 64 keys ----
+        f32x4 sacc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            sacc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < DK / 32; ++ks) {
+                const bf16x8 kf = *(const bf16x8*)(k_lds + (16 * t + col) * KSTR + (32 * ks + 8 * g) * 2);
+                sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], kf, sacc[t], 0, 0, 0);
+            }
+        }
+        // ---- mask + online softmax in base 2 (rows 4g + i, keys 16t + col) ----
+        float alpha[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int qi = row_q0 + 4 * g + i;
+            const int qpos = p0 + qi;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int kp = kt0 + 16 * t + col;
+                float v = sacc[t][i] * qs;
+                if (kp > qpos || kp < lo_row[i] || qi >= n) v = -INFINITY;
+                sacc[t][i] = v;
+                mx = fmaxf(mx, v);
+            }
+            const float mn = fmaxf(mrow[i], group_max<16>(mx));
+            alpha[i] = mn == -INFINITY ? 1.f : exp2f(mrow[i] - mn);
+            float rs = 0.f;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const float pv = mn == -INFINITY ? 0.f : exp2f(sacc[t][i] - mn);
+                sacc[t][i] = pv;
+                rs += pv;
+            }
+            lrow[i] = lrow[i] * alpha[i] + group_sum<16>(rs);
+            mrow[i] = mn;
+        }
+#pragma unroll
+        for (int nt = 0; nt < DV / 16; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oacc[nt][i] *= alpha[i];
+        // ---- P -> LDS (bf16), read back as the next A fragments by the same wave ----
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *(bf16_t*)(pw + (4 * g + i) * PSTR + (16 * t + col) * 2) = f32_to_bf16(sacc[t][i]);
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
+        __builtin_amdgcn_wave_barrier();
+        // ---- O += P V ----
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const bf16x8 pa = *(const bf16x8*)(pw + col * PSTR + (32 * ks + 8 * g) * 2);
+#pragma unroll
+            for (int nt = 0; nt < DV / 16; ++nt) {
+                const bf16x8 vb = *(const bf16x8*)(v_lds + (16 * nt + col) * VSTR + (32 * ks + 8 * g) * 2);
+                oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, oacc[nt], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int qi = row_q0 + 4 * g + i;
+        if (qi >= n) continue;
+        const float inv = lrow[i] > 0.f ? out_scale / lrow[i] : 0.f;
+#pragma unroll
+        for (int nt = 0; nt < DV / 16; ++nt) {
+            const size_t o = (size_t)qi * ldo + (size_t)hq * DV + 16 * nt + col;
+            if constexpr (O16) ((bf16_t*)out)[o] = f32_to_bf16(oacc[nt][i] * inv);
+            else ((float*)out)[o] = oacc[nt][i] * inv;
+        }
+    }
+}
+
 // grid (rows, H): combines the partitions of a row (at most 64: lane z holds partition z's maximum and sum) in a fixed
 // order; an empty partition has sum 0
 template <bool O16>
@@ -399,5 +577,39 @@ extern "C" int mxh_masked_softmax(const float* sc, void* pw, int p16, long rows,
     MXH_CHECK(sc && pw && n > 0 && nk > 0 && rows % n == 0 && rows < (1L << 31) && key0 >= 0 && p0 >= key0);
     if (p16) masked_softmax_kernel<true><<<(unsigned)rows, 256, 0, st>>>(sc, pw, n, nk, p0, key0, scale, chunk, window, sink);
     else masked_softmax_kernel<false><<<(unsigned)rows, 256, 0, st>>>(sc, pw, n, nk, p0, key0, scale, chunk, window, sink);
+    return (int)hipGetLastError();
+}
+
+// A prompt chunk of n rows of one sequence (q and out point at its first row) at positions p0 .., bf16 pools.
+// Returns hipErrorInvalidValue for head sizes without an instantiation: the caller asks mxh_attention_mfma_ok first.
+extern "C" int mxh_attention_mfma_ok(int dk, int dv) { return (dk == 64 || dk == 128) && (dv == 64 || dv == 128); }
+
+extern "C" int mxh_attention_mfma(const void* q, int ldq, const void* kc, const void* vc, int bs, const int* table,
+                                  int p0, int n, void* out, int ldo, int o16, int H, int G, int dk, int dv,
+                                  float scale, int chunk, int window, int sink, float out_scale, hipStream_t st) {
+    if (n <= 0) return 0;
+    MXH_CHECK(q && kc && vc && table && out && bs > 0 && p0 >= 0 && H > 0 && G > 0 && H % G == 0);
+    MXH_CHECK(mxh_attention_mfma_ok(dk, dv) && ldq >= H * dk && ldq % 8 == 0 && ldo >= H * dv && chunk >= 0 && window >= 0);
+    const int rep = H / G;
+    const int GW = rep % 4 == 0 ? 4 : rep % 2 == 0 ? 2 : 1;
+    const int RT = 4 / GW;
+    MXH_CHECK(H / GW <= 65535);
+    const dim3 grid((n + RT * 16 - 1) / (RT * 16), H / GW);
+#define GO(K_, V_)                                                                                                    \
+    do {                                                                                                              \
+        if (o16)                                                                                                      \
+            attn_chunk_mfma_kernel<K_, V_, true><<<grid, 256, 0, st>>>((const bf16_t*)q, ldq, (const bf16_t*)kc,       \
+                                                                       (const bf16_t*)vc, bs, table, p0, n, out, ldo, \
+                                                                       H, G, GW, scale, chunk, window, sink, out_scale); \
+        else                                                                                                          \
+            attn_chunk_mfma_kernel<K_, V_, false><<<grid, 256, 0, st>>>((const bf16_t*)q, ldq, (const bf16_t*)kc,      \
+                                                                        (const bf16_t*)vc, bs, table, p0, n, out, ldo, \
+                                                                        H, G, GW, scale, chunk, window, sink, out_scale); \
+    } while (0)
+    if (dk == 64 && dv == 64) GO(64, 64);
+    else if (dk == 64 && dv == 128) GO(64, 128);
+    else if (dk == 128 && dv == 64) GO(128, 64);
+    else GO(128, 128);
+#undef GO
     return (int)hipGetLastError();
 }

@@ -152,6 +152,9 @@ HYBRID_SIGS = {
     # q, ldq, q16, kc, vc, bs, bt, bt_stride, cu_q, ctx, n_seqs, n_rows, row_base, out, ldo, o16, H, G, dk, dv, scale,
     # chunk, window, sink, out_scale, row_off, parts, part_len, part_ml, part_o, stream
     "mxh_attention": [P, I, I, P, P, I, P, I, P, P, I, I, I, P, I, I, I, I, I, I, F, I, I, I, F, I, I, I, P, P, P],
+    # q, ldq, kc, vc, bs, table, p0, n, out, ldo, o16, H, G, dk, dv, scale, chunk, window, sink, out_scale, stream
+    "mxh_attention_mfma": [P, I, P, P, I, P, I, I, P, I, I, I, I, I, I, F, I, I, I, F, P],
+    "mxh_attention_mfma_ok": [I, I],
     # kc, vc, is16, bs, table, lo, n, G, dk, dv, kh, vh, stream
     "mxh_kv_gather": [P, P, I, I, P, I, I, I, I, I, P, P, P],
     # src, s16, s_stride_i, s_stride_h, dst, d16, d_stride_i, d_stride_h, n, H, d, scale, stream

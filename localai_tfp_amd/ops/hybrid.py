@@ -141,7 +141,8 @@ def _attn_ref(q, kc, vc, table, ctx, pos0, H, G, dk, dv, scale, chunk, window, s
     out.copy_((o.reshape(n, H * dv) * out_scale).to(out.dtype))
 
 
-GEMM_MIN_ROWS = 64  # prompt chunks of at least this many rows take the library-GEMM route (GPU)
+MFMA_MIN_ROWS = 16  # bf16 prompt chunks of at least this many rows take the matrix-core kernel (head sizes 64 / 128)
+GEMM_MIN_ROWS = 64  # other prompt chunks of at least this many rows take the library-GEMM route (GPU)
 GEMM_MAX_SCORES = 1 << 26  # fp32 scores of one sub-problem of that route
 DECODE_WAVES = 4096  # decode rows: waves to aim for when splitting contexts into key partitions
 
@@ -211,8 +212,9 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
 
     On the GPU decode rows and short chunks run the row kernel (one wave per row and head; decode rows split their
     visible keys into partitions merged through `workspace` = (fp32 [rows, 2], fp32 [rows, dv]), rows >= n_dec * H
-    * partitions); chunks of GEMM_MIN_ROWS rows and more, when the step's chunk sizes are known on the host, run as
-    library GEMMs around a masked softmax kernel."""
+    * partitions). When the step's chunk sizes are known on the host, bf16 chunks of MFMA_MIN_ROWS rows and more with
+    head sizes of 64 or 128 run on the matrix-core kernel, and other chunks of GEMM_MIN_ROWS rows and more as library
+    GEMMs around a masked softmax kernel."""
     T = q.shape[0]
     if T == 0:
         return out
@@ -262,17 +264,26 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
             N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
                     rag.pf_bt.data_ptr(), rag.pf_bt.stride(0), rag.pf_cu.data_ptr(), rag.pf_ctx.data_ptr(), rag.n_pf,
                     n_rows, nd, out.data_ptr(), out.stride(0), _is16(out), *common, row_off, 1, 0, None, None, st)
-        if lens is None or max(lens) < GEMM_MIN_ROWS or 0 < chunk < GEMM_MIN_ROWS:
+        mfma = q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and MFMA_MIN_ROWS > 0 and \
+            bool(N.hybrid_kernels().mxh_attention_mfma_ok(dk, dv))
+        big = MFMA_MIN_ROWS if mfma else GEMM_MIN_ROWS
+        if lens is None or max(lens) < big or (not mfma and 0 < chunk < GEMM_MIN_ROWS):
             rows_kernel(0, T - nd)  # (chunks shorter than a block of rows: a row's few visible keys suit the row kernel)
             return out
         r, run0 = 0, None  # run0: first row of a run of consecutive short chunks
         for k, n in enumerate(lens):
-            if n >= GEMM_MIN_ROWS:
+            if n >= big:
                 if run0 is not None:
                     rows_kernel(run0, r - run0)
                     run0 = None
-                _attn_gemm_chunk(q[nd + r:nd + r + n], kc, vc, rag.pf_bt[k], rag.pf_ctx_host[k] - n, n, H, G, dk, dv,
-                                 scale, chunk, window, sink, out[nd + r:nd + r + n], out_scale)
+                qk, ok = q[nd + r:nd + r + n], out[nd + r:nd + r + n]
+                if mfma:
+                    N.kcall("mxh_attention_mfma", qk.data_ptr(), qk.stride(0), kc.data_ptr(), vc.data_ptr(), bs,
+                            rag.pf_bt[k].data_ptr(), rag.pf_ctx_host[k] - n, n, ok.data_ptr(), ok.stride(0), _is16(out),
+                            H, G, dk, dv, float(scale), int(chunk), int(window), int(sink), float(out_scale), st)
+                else:
+                    _attn_gemm_chunk(qk, kc, vc, rag.pf_bt[k], rag.pf_ctx_host[k] - n, n, H, G, dk, dv, scale, chunk,
+                                     window, sink, ok, out_scale)
             elif n and run0 is None:
                 run0 = r
             r += n

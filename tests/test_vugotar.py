@@ -216,6 +216,15 @@ def test_attention_chunk_edges_pages_and_sink(dev, dt, tol, gemm_rows, monkeypat
     close(got, want, tol)
     got, want = _attention_case(dev, dt, 2, 2, 64, 72, 64, 0, 90, [50, 40], 8, 0.3)  # no chunks: plain causal
     close(got, want, tol)
+    # head sizes of 64 and 128 (the matrix-core kernel takes bf16 portions of 16 rows and more): four, two and one
+    # query heads per key head, dim != vdim, portions that start and end inside 16-row tiles, pages and chunks
+    plant = [(79, 40), (119, 80), (120, 119), (121, 120), (95, 81), (149, 127), (60, 60), (39, 0), (41, 39)]
+    for H, G, dk, dv, rot, ch in ((4, 2, 64, 64, 0, 40), (8, 2, 128, 128, 0, 40), (2, 2, 64, 128, 0, 40),
+                                  (6, 3, 128, 64, 0, 40)):
+        got, want = _attention_case(dev, dt, H, G, dk, dv, rot, ch, 150, [37, 2, 41, 1, 17, 22, 1, 29], bs, 0.5, plant)
+        close(got, want, tol * (4 if dt == "bfloat16" else 1))
+    got, want = _attention_case(dev, dt, 4, 1, 64, 64, 32, 0, 200, [130, 70], 16, 0.2)  # rotated, plain causal
+    close(got, want, tol)
     # rows decoded alone behind 260 and more visible keys: their keys are split into partitions and merged
     plant = [(270, 3), (280, 127), (281, 128), (299, 255), (290, 256), (295, 295)]
     got, want = _attention_case(dev, dt, 2, 1, 16, 16, 16, 0, 300, [200, 60] + [1] * 40, 16, 3.0, plant)
