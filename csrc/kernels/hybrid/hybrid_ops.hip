@@ -26,7 +26,7 @@ MX_DEV float silu_acc(float x) { return x / (1.f + expf(-x)); }
 MX_DEV float sigmoid_acc(float x) { return 1.f / (1.f + expf(-x)); }
 MX_DEV float softplus_acc(float x) { return x > 30.f ? x : log1pf(expf(x)); }
 
-// sum over the threads of a block of blockDim.x = 64 * k threads (k <= 4), returned to every thread
+// sum over the threads of a block of blockDim.x = 64 * k threads (k <= 16), returned to every thread
 MX_DEV float block_sum_dyn(float v, float* red) {
     v = wave_sum(v);
     const int nw = blockDim.x >> 6;
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(NT) void scan_coefs_kernel(const float* a, int lda,
 template <bool B16, int GC>
 __global__ void gated_group_norm_kernel(const float* y, int ldy, const float* gate, int ldg, const float* w, int wlen,
                                         float eps, int group, int gate_first, float out_scale, void* out, int ldo) {
-    __shared__ float red[NT / 64];
+    __shared__ float red[16];
     const int t = blockIdx.x, c0 = blockIdx.y * group;
     const float* yr = y + (long)t * ldy + c0;
     const float* gr = gate + (long)t * ldg + c0;
@@ -485,7 +485,8 @@ extern "C" int mxh_gated_group_norm(const float* y, int ldy, const float* gate, 
     do {                                     \
         if (group <= 256) GO(B, 4, 64);      \
         else if (group <= 2048) GO(B, 8, NT); \
-        else GO(B, 32, NT);                  \
+        else if (group <= 8192) GO(B, 8, 1024); \
+        else GO(B, 32, 1024);                \
     } while (0)
     if (o16) PICK(true);
     else PICK(false);
