@@ -46,7 +46,7 @@ MX_DEV void dot_row(const void* base, long off, const float* q, int n, float (&a
             const int m = n / 8;
             int i = 0;
             for (; i + 8 <= m; i += 8) {
-                uint4 w[8];
+                uint4 w[8];  // (a struct type: kept in registers here only because every index is a constant after unrolling)
 #pragma unroll
                 for (int e = 0; e < 8; ++e) w[e] = p[i + e];
 #pragma unroll
@@ -230,13 +230,68 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
     }
 }
 
+// Staging of a key tile [KT][DK] and a value tile [KT][DV] (both row-major, padded rows) by NTH threads: 16-byte pieces wait in
+// registers (tile_load) until the previous tile has been worked on, then go to LDS (tile_store). Plain functions over
+// array references: the pieces stay in registers.
+template <int DK, int DV, int KT, int NTH>
+MX_DEV void tile_load(u32x4 (&kr)[KT * DK / 8 / NTH], u32x4 (&vr)[KT * DV / 8 / NTH], const bf16_t* __restrict__ kc,
+                      const bf16_t* __restrict__ vc, const int* __restrict__ table, int bs, int G, int kvh, int kt0,
+                      int kv_end, int tid) {
+#pragma unroll
+    for (int j = 0; j < KT * DK / 8 / NTH; ++j) {
+        const int id = tid + j * NTH;
+        const int p = id / (DK / 8), c = id % (DK / 8);
+        const int pos = min(kt0 + p, kv_end - 1);  // clamped: keys past the end are masked by the caller
+        const size_t tok = (size_t)table[pos / bs] * bs + (pos % bs);
+        kr[j] = *(const u32x4*)(kc + (tok * G + kvh) * DK + c * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < KT * DV / 8 / NTH; ++j) {
+        const int id = tid + j * NTH;
+        const int p = id / (DV / 8), c = id % (DV / 8);
+        const int pos = min(kt0 + p, kv_end - 1);
+        const size_t tok = (size_t)table[pos / bs] * bs + (pos % bs);
+        vr[j] = *(const u32x4*)(vc + (tok * G + kvh) * DV + c * 8);
+    }
+}
+template <int DK, int DV, int KT, int NTH, int KSTR, int VSTR>
+MX_DEV void tile_store(const u32x4 (&kr)[KT * DK / 8 / NTH], const u32x4 (&vr)[KT * DV / 8 / NTH], char* k_lds,
+                       char* v_lds, int tid) {
+#pragma unroll
+    for (int j = 0; j < KT * DK / 8 / NTH; ++j) {
+        const int id = tid + j * NTH;
+        const int p = id / (DK / 8), c = id % (DK / 8);
+        *(u32x4*)(k_lds + p * KSTR + c * 16) = kr[j];
+    }
+#pragma unroll
+    for (int j = 0; j < KT * DV / 8 / NTH; ++j) {
+        const int id = tid + j * NTH;
+        const int p = id / (DV / 8), c = id % (DV / 8);
+        *(u32x4*)(v_lds + p * VSTR + c * 16) = vr[j];
+    }
+}
+
+// B fragment of O += P V from a row-major value tile in LDS (row = key, VSTR bytes apart): the values of keys
+// r0 .. r0 + 7 at dim 16 nt + col, through the transposing LDS read (each lane of a 16-lane group hands in 4 dims of one
+// key and receives one dim of 4 keys). The result is reinterpreted as a whole vector.
+template <int VSTR>
+MX_DEV bf16x8 v_fragment(const char* v_lds, int r0, int nt, int col) {
+    const int q4 = col >> 2, p4 = col & 3;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MX_LDS s16x4*)(v_lds + (r0 + q4) * VSTR + 32 * nt + 8 * p4));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MX_LDS s16x4*)(v_lds + (r0 + 4 + q4) * VSTR + 32 * nt + 8 * p4));
+    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+    const u32x4 w4 = {l2[0], l2[1], h2[0], h2[1]};
+    return __builtin_bit_cast(bf16x8, w4);
+}
+
 // attn_chunk_mfma_kernel: a prompt chunk of one sequence on the matrix cores (bf16 pools, head sizes that are
 // multiples of 32 / 16). A workgroup of 4 waves owns RT 16-row query tiles of GW query heads that share a key / value
 // head (GW * RT = 4); a wave owns one tile of one head, its query fragments in registers. Keys are taken 64 at a time:
-// the workgroup stages the key tile [64][DK] and the transposed value tile [DV][64] in LDS (the next tile's numbers are
+// the workgroup stages the key tile [64][DK] and the value tile [64][DV] in LDS (the next tile's numbers are
 // requested from memory before the current tile is worked on and wait in registers), each wave forms S = Q K^T with
 // MFMA 16x16x32, masks (causal, chunk or window start) and updates its rows' running maximum and sum in fp32 (the sink
-// starts them at 0 and 1), writes the weights as bf16 to its own LDS patch and accumulates O += P V.
+// starts them at 0 and 1), writes the weights as bf16 to its own LDS patch and accumulates O += P V, the value
+// fragments coming out of LDS through the transposing read.
 // Fragment layout of v_mfma_f32_16x16x32_bf16 (g = lane / 16, col = lane % 16): A holds row col, k = 8g .. 8g + 7;
 // B holds column col, k = 8g .. 8g + 7; the result holds rows 4g .. 4g + 3 of column col.
 template <int DK, int DV, bool O16>
@@ -248,11 +303,11 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
                                                               int window, int sink, float out_scale) {
     constexpr int KT = 64;
     constexpr int KSTR = (DK + 8) * 2;  // bytes per key row in LDS (padded)
-    constexpr int VSTR = (KT + 8) * 2;  // bytes per transposed value row (one dim, 64 keys)
+    constexpr int VSTR = (DV + 8) * 2;  // bytes per value row in LDS (padded)
     constexpr int PSTR = (KT + 8) * 2;  // bytes per weight row
     constexpr float LOG2E_ = 1.4426950408889634f;
     __shared__ __attribute__((aligned(16))) char k_lds[KT * KSTR];
-    __shared__ __attribute__((aligned(16))) char v_lds[DV * VSTR];
+    __shared__ __attribute__((aligned(16))) char v_lds[KT * VSTR];
     __shared__ __attribute__((aligned(16))) char p_lds[4 * 16 * PSTR];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int g = lane >> 4, col = lane & 15;
@@ -291,46 +346,13 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
     char* pw = p_lds + wave * 16 * PSTR;
 
     constexpr int KCH = KT * DK / 8 / 256, VCH = KT * DV / 8 / 256;  // 16-byte pieces per thread
-    uint4 kr[KCH], vr[VCH];
-    auto load_tile = [&](int kt0) {
-#pragma unroll
-        for (int j = 0; j < KCH; ++j) {
-            const int id = threadIdx.x + j * 256;
-            const int p = id / (DK / 8), c = id % (DK / 8);
-            const int pos = min(kt0 + p, kv_end - 1);  // clamped: keys past the end are masked below
-            const size_t tok = (size_t)table[pos / bs] * bs + (pos % bs);
-            kr[j] = *(const uint4*)(kc + (tok * G + kvh) * DK + c * 8);
-        }
-#pragma unroll
-        for (int j = 0; j < VCH; ++j) {
-            const int id = threadIdx.x + j * 256;
-            const int p = id / (DV / 8), c = id % (DV / 8);
-            const int pos = min(kt0 + p, kv_end - 1);
-            const size_t tok = (size_t)table[pos / bs] * bs + (pos % bs);
-            vr[j] = *(const uint4*)(vc + (tok * G + kvh) * DV + c * 8);
-        }
-    };
-    auto store_tile = [&]() {
-#pragma unroll
-        for (int j = 0; j < KCH; ++j) {
-            const int id = threadIdx.x + j * 256;
-            const int p = id / (DK / 8), c = id % (DK / 8);
-            *(uint4*)(k_lds + p * KSTR + c * 16) = kr[j];
-        }
-#pragma unroll
-        for (int j = 0; j < VCH; ++j) {
-            const int id = threadIdx.x + j * 256;
-            const int p = id / (DV / 8), c = id % (DV / 8);
-            const uint32_t w[4] = {vr[j].x, vr[j].y, vr[j].z, vr[j].w};
-#pragma unroll
-            for (int jj = 0; jj < 8; ++jj)
-                *(bf16_t*)(v_lds + (8 * c + jj) * VSTR + 2 * p) = (bf16_t)(w[jj >> 1] >> (16 * (jj & 1)));
-        }
-    };
-    if (kt_begin < kv_end) load_tile(kt_begin);
+    u32x4 kr[KCH], vr[VCH];
+#define LOAD_TILE(kt0_) tile_load<DK, DV, KT, 256>(kr, vr, kc, vc, table, bs, G, kvh, kt0_, kv_end, threadIdx.x)
+#define STORE_TILE() tile_store<DK, DV, KT, 256, KSTR, VSTR>(kr, vr, k_lds, v_lds, threadIdx.x)
+    if (kt_begin < kv_end) LOAD_TILE(kt_begin);
     for (int kt0 = kt_begin; kt0 < kv_end; kt0 += KT) {
-        store_tile();
-        if (kt0 + KT < kv_end) load_tile(kt0 + KT);
+        STORE_TILE();
+        if (kt0 + KT < kv_end) LOAD_TILE(kt0 + KT);
         __syncthreads();
         // ---- S = Q K^T : 16 rows x 64 keys ----
         f32x4 sacc[4];
@@ -387,10 +409,9 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
         for (int ks = 0; ks < 2; ++ks) {
             const bf16x8 pa = *(const bf16x8*)(pw + col * PSTR + (32 * ks + 8 * g) * 2);
 #pragma unroll
-            for (int nt = 0; nt < DV / 16; ++nt) {
-                const bf16x8 vb = *(const bf16x8*)(v_lds + (16 * nt + col) * VSTR + (32 * ks + 8 * g) * 2);
-                oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, oacc[nt], 0, 0, 0);
-            }
+            for (int nt = 0; nt < DV / 16; ++nt)
+                oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, v_fragment<VSTR>(v_lds, 32 * ks + 8 * g, nt, col),
+                                                                   oacc[nt], 0, 0, 0);
         }
         __syncthreads();
     }
@@ -407,6 +428,169 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
         }
     }
 }
+
+// attn_decode_mfma_kernel: single new tokens on the matrix cores (bf16 pools, head sizes 64 / 128, up to 16 query heads
+// per key / value head). grid (sequences, G, partitions), one wave per workgroup: the 16 rows of its tile are the
+// query heads that share key / value head blockIdx.y (rows beyond H / G are zero), all at the sequence's newest
+// position, so a key and value tile is read once for all of them. The wave walks its partition's keys
+// as attn_chunk_mfma_kernel does, 32 at a time (key fragments straight from the pages, values staged in LDS by the
+// wave itself, the next tile requested ahead). With one
+// partition it writes the result, otherwise (max, sum, unnormalised output) for attn_merge_kernel; the running maximum
+// is kept in base 2 and handed over in base e.
+template <int DK, int DV, bool O16>
+__global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __restrict__ q, int ldq,
+                                                              const bf16_t* __restrict__ kc,
+                                                              const bf16_t* __restrict__ vc, int bs,
+                                                              const int* __restrict__ bt, int bt_stride,
+                                                              const int* __restrict__ ctx, void* out, int ldo, int H,
+                                                              int G, float scale, int chunk, int window, int sink,
+                                                              float out_scale, int parts, int part_len,
+                                                              float* __restrict__ part_ml, float* __restrict__ part_o) {
+    constexpr int KT = 32;  // keys per tile: the wave stages its tiles alone, 64 keys would not fit its registers
+    constexpr int VSTR = (DV + 8) * 2, PSTR = (KT + 8) * 2;
+    constexpr float LOG2E_ = 1.4426950408889634f, LN2_ = 0.6931471805599453f;
+    __shared__ __attribute__((aligned(16))) char v_lds[KT * VSTR];
+    __shared__ __attribute__((aligned(16))) char pw[16 * PSTR];
+    const int lane = threadIdx.x, g = lane >> 4, col = lane & 15;
+    const int s = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
+    const int rep = H / G;
+    const int qpos = ctx[s] - 1;
+    int lo = chunk > 0 ? (qpos / chunk) * chunk : window > 0 ? max(0, qpos - window + 1) : 0;
+    int kv_end = qpos + 1;
+    if (parts > 1) {
+        lo += z * part_len;
+        kv_end = min(kv_end, lo + part_len);
+        sink = 0;  // joins in the merge
+    }
+    const int* table = bt + (size_t)s * bt_stride;
+    const float qs = scale * LOG2E_;
+    bf16x8 qf[DK / 32];
+    {
+        const bf16_t* qp = q + (size_t)s * ldq + (size_t)(kvh * rep + min(col, rep - 1)) * DK + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < DK / 32; ++ks) {
+            const uint4 w = *(const uint4*)(qp + 32 * ks);
+            const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+            qf[ks] = __builtin_bit_cast(bf16x8, col < rep ? w : zero);
+        }
+    }
+    f32x4 oacc[DV / 16];
+#pragma unroll
+    for (int i = 0; i < DV / 16; ++i) oacc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float mrow[4], lrow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        mrow[i] = sink ? 0.f : -INFINITY;
+        lrow[i] = sink ? 1.f : 0.f;
+    }
+    // key fragments come straight from the pages (lane (g, col) of tile t: key 16 t + col, dims 32 ks + 8 g .. + 7 are 16
+    // contiguous bytes); values are staged row-major in LDS. Both are requested one tile ahead.
+    constexpr int VCH = KT * DV / 8 / 64;  // 16-byte value pieces per lane
+    u32x4 kf[KT / 16][DK / 32], vr[VCH];
+    auto load_tile = [&](int kt0) {
+#pragma unroll
+        for (int t = 0; t < KT / 16; ++t) {
+            const int pos = min(kt0 + 16 * t + col, kv_end - 1);  // clamped: keys past the end are masked below
+            const bf16_t* kp = kc + (((size_t)table[pos / bs] * bs + (pos % bs)) * G + kvh) * DK + 8 * g;
+#pragma unroll
+            for (int ks = 0; ks < DK / 32; ++ks) kf[t][ks] = *(const u32x4*)(kp + 32 * ks);
+        }
+#pragma unroll
+        for (int j = 0; j < VCH; ++j) {
+            const int id = lane + j * 64;
+            const int p = id / (DV / 8), c = id % (DV / 8);
+            const int pos = min(kt0 + p, kv_end - 1);
+            vr[j] = *(const u32x4*)(vc + (((size_t)table[pos / bs] * bs + (pos % bs)) * G + kvh) * DV + c * 8);
+        }
+    };
+    if (lo < kv_end) load_tile(lo);
+    for (int kt0 = lo; kt0 < kv_end; kt0 += KT) {
+        __syncthreads();  // (one wave: orders the previous tile's LDS reads before these writes)
+#pragma unroll
+        for (int j = 0; j < VCH; ++j) {
+            const int id = lane + j * 64;
+            *(u32x4*)(v_lds + (id / (DV / 8)) * VSTR + (id % (DV / 8)) * 16) = vr[j];
+        }
+        f32x4 sacc[KT / 16];
+#pragma unroll
+        for (int t = 0; t < KT / 16; ++t) {
+            sacc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < DK / 32; ++ks)
+                sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], __builtin_bit_cast(bf16x8, kf[t][ks]), sacc[t],
+                                                                  0, 0, 0);
+        }
+        if (kt0 + KT < kv_end) load_tile(kt0 + KT);
+        float alpha[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < KT / 16; ++t) {
+                const int kp = kt0 + 16 * t + col;
+                float v = sacc[t][i] * qs;
+                if (kp >= kv_end) v = -INFINITY;
+                sacc[t][i] = v;
+                mx = fmaxf(mx, v);
+            }
+            const float mn = fmaxf(mrow[i], group_max<16>(mx));
+            alpha[i] = mn == -INFINITY ? 1.f : exp2f(mrow[i] - mn);
+            float rs = 0.f;
+#pragma unroll
+            for (int t = 0; t < KT / 16; ++t) {
+                const float pv = mn == -INFINITY ? 0.f : exp2f(sacc[t][i] - mn);
+                sacc[t][i] = pv;
+                rs += pv;
+            }
+            lrow[i] = lrow[i] * alpha[i] + group_sum<16>(rs);
+            mrow[i] = mn;
+        }
+#pragma unroll
+        for (int nt = 0; nt < DV / 16; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oacc[nt][i] *= alpha[i];
+#pragma unroll
+        for (int t = 0; t < KT / 16; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *(bf16_t*)(pw + (4 * g + i) * PSTR + (16 * t + col) * 2) = f32_to_bf16(sacc[t][i]);
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < KT / 32; ++ks) {
+            const bf16x8 pa = *(const bf16x8*)(pw + col * PSTR + (32 * ks + 8 * g) * 2);
+#pragma unroll
+            for (int nt = 0; nt < DV / 16; ++nt)
+                oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, v_fragment<VSTR>(v_lds, 32 * ks + 8 * g, nt, col),
+                                                                   oacc[nt], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = 4 * g + i;
+        if (r >= rep) continue;
+        const int h = kvh * rep + r;
+        if (parts > 1) {
+            const size_t pr = ((size_t)s * H + h) * parts + z;
+            if (col == 0) {
+                part_ml[pr * 2] = mrow[i] * LN2_;
+                part_ml[pr * 2 + 1] = lrow[i];
+            }
+#pragma unroll
+            for (int nt = 0; nt < DV / 16; ++nt) part_o[pr * DV + 16 * nt + col] = oacc[nt][i];
+            continue;
+        }
+        const float inv = lrow[i] > 0.f ? out_scale / lrow[i] : 0.f;
+#pragma unroll
+        for (int nt = 0; nt < DV / 16; ++nt) {
+            const size_t o = (size_t)s * ldo + (size_t)h * DV + 16 * nt + col;
+            if constexpr (O16) ((bf16_t*)out)[o] = f32_to_bf16(oacc[nt][i] * inv);
+            else ((float*)out)[o] = oacc[nt][i] * inv;
+        }
+    }
+}
+
+#undef LOAD_TILE
+#undef STORE_TILE
 
 // grid (rows, H): combines the partitions of a row (at most 64: lane z holds partition z's maximum and sum) in a fixed
 // order; an empty partition has sum 0
@@ -611,5 +795,41 @@ extern "C" int mxh_attention_mfma(const void* q, int ldq, const void* kc, const 
     else if (dk == 128 && dv == 64) GO(128, 64);
     else GO(128, 128);
 #undef GO
+    return (int)hipGetLastError();
+}
+
+// Decode rows (row r = sequence r's new token) on the matrix cores; same conditions as mxh_attention_mfma plus at most
+// 16 query heads per key / value head. Partitions as in mxh_attention.
+extern "C" int mxh_attention_decode_mfma(const void* q, int ldq, const void* kc, const void* vc, int bs, const int* bt,
+                                         int bt_stride, const int* ctx, int n_seqs, void* out, int ldo, int o16, int H,
+                                         int G, int dk, int dv, float scale, int chunk, int window, int sink,
+                                         float out_scale, int parts, int part_len, float* part_ml, float* part_o,
+                                         hipStream_t st) {
+    if (n_seqs <= 0) return 0;
+    MXH_CHECK(q && kc && vc && bt && ctx && out && bs > 0 && bt_stride > 0 && H > 0 && G > 0 && H % G == 0);
+    MXH_CHECK(H / G <= 16 && G <= 65535 && mxh_attention_mfma_ok(dk, dv) && ldq >= H * dk && ldq % 8 == 0 && ldo >= H * dv);
+    MXH_CHECK(parts >= 1 && parts <= 64 && (parts == 1 || (part_len > 0 && part_ml && part_o)) && chunk >= 0 && window >= 0);
+    const dim3 grid(n_seqs, G, parts);
+#define GO(K_, V_)                                                                                                       \
+    do {                                                                                                                 \
+        if (o16)                                                                                                         \
+            attn_decode_mfma_kernel<K_, V_, true><<<grid, 64, 0, st>>>(                                                  \
+                (const bf16_t*)q, ldq, (const bf16_t*)kc, (const bf16_t*)vc, bs, bt, bt_stride, ctx, out, ldo, H, G, scale, \
+                chunk, window, sink, out_scale, parts, part_len, part_ml, part_o);                                       \
+        else                                                                                                             \
+            attn_decode_mfma_kernel<K_, V_, false><<<grid, 64, 0, st>>>(                                                 \
+                (const bf16_t*)q, ldq, (const bf16_t*)kc, (const bf16_t*)vc, bs, bt, bt_stride, ctx, out, ldo, H, G, scale, \
+                chunk, window, sink, out_scale, parts, part_len, part_ml, part_o);                                       \
+    } while (0)
+    if (dk == 64 && dv == 64) GO(64, 64);
+    else if (dk == 64 && dv == 128) GO(64, 128);
+    else if (dk == 128 && dv == 64) GO(128, 64);
+    else GO(128, 128);
+#undef GO
+    if (parts > 1) {
+        const dim3 g2(n_seqs, H);
+        if (o16) attn_merge_kernel<true><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, 0, out, ldo);
+        else attn_merge_kernel<false><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, 0, out, ldo);
+    }
     return (int)hipGetLastError();
 }

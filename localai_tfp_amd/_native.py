@@ -155,6 +155,9 @@ HYBRID_SIGS = {
     # q, ldq, kc, vc, bs, table, p0, n, out, ldo, o16, H, G, dk, dv, scale, chunk, window, sink, out_scale, stream
     "mxh_attention_mfma": [P, I, P, P, I, P, I, I, P, I, I, I, I, I, I, F, I, I, I, F, P],
     "mxh_attention_mfma_ok": [I, I],
+    # q, ldq, kc, vc, bs, bt, bt_stride, ctx, n_seqs, out, ldo, o16, H, G, dk, dv, scale, chunk, window, sink, out_scale,
+    # parts, part_len, part_ml, part_o, stream
+    "mxh_attention_decode_mfma": [P, I, P, P, I, P, I, P, I, P, I, I, I, I, I, I, F, I, I, I, F, I, I, P, P, P],
     # kc, vc, is16, bs, table, lo, n, G, dk, dv, kh, vh, stream
     "mxh_kv_gather": [P, P, I, I, P, I, I, I, I, I, P, P, P],
     # src, s16, s_stride_i, s_stride_h, dst, d16, d_stride_i, d_stride_h, n, H, d, scale, stream

@@ -212,9 +212,9 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
 
     On the GPU decode rows and short chunks run the row kernel (one wave per row and head; decode rows split their
     visible keys into partitions merged through `workspace` = (fp32 [rows, 2], fp32 [rows, dv]), rows >= n_dec * H
-    * partitions). When the step's chunk sizes are known on the host, bf16 chunks of MFMA_MIN_ROWS rows and more with
-    head sizes of 64 or 128 run on the matrix-core kernel, and other chunks of GEMM_MIN_ROWS rows and more as library
-    GEMMs around a masked softmax kernel."""
+    * partitions). bf16 tensors with head sizes of 64 or 128 run on the matrix cores: decode rows (up to 16 query
+    heads per key head) and, when the step's chunk sizes are known on the host, chunks of MFMA_MIN_ROWS rows and more.
+    Other chunks of GEMM_MIN_ROWS rows and more run as library GEMMs around a masked softmax kernel."""
     T = q.shape[0]
     if T == 0:
         return out
@@ -241,22 +241,31 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
     bs = kc.shape[1]
     st = N.stream_ptr()
     common = (H, G, dk, dv, float(scale), int(chunk), int(window), int(sink), float(out_scale))
+    mfma_ok = q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and MFMA_MIN_ROWS > 0 and \
+        bool(N.hybrid_kernels().mxh_attention_mfma_ok(dk, dv))
     if nd:
         vis = rag.dec_max_len
         vis = min(vis, chunk) if chunk else min(vis, window) if window else vis
+        dec_mfma = mfma_ok and H // G <= 16  # a wave's 16 rows are the query heads of one key / value head
         parts, plen = 1, 0
         if workspace is not None:
-            plen = decode_part_len(nd, H, vis)
+            plen = decode_part_len(nd, G * 4 if dec_mfma else H, vis)
             parts = -(-vis // plen)
             room = min(64, workspace[0].shape[0] // (nd * H))  # the merge holds one partition per lane
             if parts > room:
                 parts = max(1, room)
                 plen = -(-(-(-vis // parts)) // 64) * 64
         ml, po = (workspace[0], workspace[1]) if parts > 1 else (None, None)
-        N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
-                rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), None, rag.dec_lens.data_ptr(), nd, nd, 0,
-                out.data_ptr(), out.stride(0), _is16(out), *common, 0, parts, plen if parts > 1 else 0, N.ptr(ml),
-                N.ptr(po), st)
+        if dec_mfma:
+            N.kcall("mxh_attention_decode_mfma", q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), bs,
+                    rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), rag.dec_lens.data_ptr(), nd, out.data_ptr(),
+                    out.stride(0), _is16(out), H, G, dk, dv, float(scale), int(chunk), int(window), int(sink),
+                    float(out_scale), parts, plen if parts > 1 else 0, N.ptr(ml), N.ptr(po), st)
+        else:
+            N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
+                    rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), None, rag.dec_lens.data_ptr(), nd, nd, 0,
+                    out.data_ptr(), out.stride(0), _is16(out), *common, 0, parts, plen if parts > 1 else 0, N.ptr(ml),
+                    N.ptr(po), st)
     if rag.n_pf:
         lens = rag.pf_q_host if len(rag.pf_q_host) == rag.n_pf and len(rag.pf_ctx_host) == rag.n_pf else None
 
@@ -264,8 +273,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
             N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
                     rag.pf_bt.data_ptr(), rag.pf_bt.stride(0), rag.pf_cu.data_ptr(), rag.pf_ctx.data_ptr(), rag.n_pf,
                     n_rows, nd, out.data_ptr(), out.stride(0), _is16(out), *common, row_off, 1, 0, None, None, st)
-        mfma = q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and MFMA_MIN_ROWS > 0 and \
-            bool(N.hybrid_kernels().mxh_attention_mfma_ok(dk, dv))
+        mfma = mfma_ok
         big = MFMA_MIN_ROWS if mfma else GEMM_MIN_ROWS
         if lens is None or max(lens) < big or (not mfma and 0 < chunk < GEMM_MIN_ROWS):
             rows_kernel(0, T - nd)  # (chunks shorter than a block of rows: a row's few visible keys suit the row kernel)

@@ -229,6 +229,10 @@ def test_attention_chunk_edges_pages_and_sink(dev, dt, tol, gemm_rows, monkeypat
     plant = [(270, 3), (280, 127), (281, 128), (299, 255), (290, 256), (295, 295)]
     got, want = _attention_case(dev, dt, 2, 1, 16, 16, 16, 0, 300, [200, 60] + [1] * 40, 16, 3.0, plant)
     close(got, want, tol * (4 if dt == "bfloat16" else 1))
+    got, want = _attention_case(dev, dt, 4, 1, 64, 64, 64, 0, 300, [200, 60] + [1] * 40, 16, 1.0, plant)  # matrix cores
+    close(got, want, tol * (4 if dt == "bfloat16" else 1))
+    got, want = _attention_case(dev, dt, 6, 2, 128, 64, 0, 0, 300, [259] + [1] * 41, 16, 0.5, plant)
+    close(got, want, tol * (4 if dt == "bfloat16" else 1))
 
 
 @pytest.mark.parametrize("dev", DEVS)
