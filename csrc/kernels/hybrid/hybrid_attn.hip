@@ -10,7 +10,10 @@
 // With parts > 1 (decode rows of long contexts) grid.z splits a row's visible keys into partitions whose
 // (max, sum, unnormalised output) go to a workspace; attn_merge_kernel combines them in a fixed order and adds the sink.
 //
-// Long prompt chunks take another route (ops/hybrid.py): kv_gather_kernel copies the chunk's visible keys and values
+// bf16 pools with head sizes of 64 / 128 run on the matrix cores instead: attn_chunk_mfma_kernel for prompt chunks,
+// attn_decode_mfma_kernel for single new tokens (both further down, with their fragment layouts).
+//
+// Other long prompt chunks take another route (ops/hybrid.py): kv_gather_kernel copies the chunk's visible keys and values
 // from the pages into head-major matrices, head_transpose_kernel does the same for the queries, the library computes
 // the score and value products, and masked_softmax_kernel turns raw scores into masked, sink-normalised weights.
 #include "../mx_common.h"
