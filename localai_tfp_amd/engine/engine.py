@@ -410,8 +410,13 @@ class LLMEngine:
             self.kv = model.make_state_cache(nb, c.block_size)
         elif self.latent:
             # the model says how many pool numbers one token takes in each of its cached layers
-            nb = c.num_blocks or LatentCache.auto_num_blocks(model.cache_ranks(), c.block_size, self.device, frac,
-                                                             dtype_bytes=model.dtype.itemsize)
+            ranks = model.cache_ranks()
+            if c.num_blocks:
+                nb = c.num_blocks
+            elif ranks:
+                nb = LatentCache.auto_num_blocks(ranks, c.block_size, self.device, frac, dtype_bytes=model.dtype.itemsize)
+            else:  # no layer keeps anything per token (recurrent layers only): blocks are bookkeeping, every sequence
+                nb = self.max_blocks_per_seq * c.max_num_seqs + 1  # may grow to the full length
             self.kv = model.make_cache(nb, c.block_size, c.max_num_seqs)
             self.state_slots = SlotPool(c.max_num_seqs)
         else:

@@ -401,6 +401,24 @@ def test_prompt_portions_and_decoding(dev, dt, tol, shape):
 
 
 @pytest.mark.parametrize("dev,dt,tol", RUNS)
+def test_recurrent_layers_only(dev, dt, tol):
+    """A model without any attention layer: the paged pool is empty, blocks are bookkeeping only (the engine sizes
+    them without a pool), states and tails carry everything."""
+    kw = dict(SHAPES["plain"], pattern=("mamba2", "mamba2", "mamba2"), mlps=("dense", None, "moe"), loop=(1, 3, 2))
+    cfg, tensors, model = build(dev, dt, seed=13, **kw)
+    assert model.cache_ranks() == []
+    t = toks(60, cfg.vocab, 3)
+    want = oracle(cfg, tensors, t)
+    ec = EngineConfig(max_num_seqs=2, max_batched_tokens=64, max_model_len=64, block_size=16, use_graphs=False,
+                      overlap=False, native_scheduler=False, logits_rows=64, gemm_autotune=False)
+    eng = LLMEngine(model, ByteTokenizer(cfg.vocab), ec)
+    assert eng.bm.num_blocks == 2 * 4 + 1
+    b16 = dt == "bfloat16"
+    close(run_cuts(eng, "a", t, [60]), want, tol / 2 if b16 else tol, b16)
+    close(run_cuts(eng, "b", t, [7, 2, 30] + [1] * 21), want, tol / 2 if b16 else tol, b16)
+
+
+@pytest.mark.parametrize("dev,dt,tol", RUNS)
 def test_residual_after_every_layer_run(dev, dt, tol):
     """The residual stream after each run of a layer (a looped layer counts every pass)."""
     cfg, tensors, model = build(dev, dt, seed=9, **SHAPES["plain"])
