@@ -607,3 +607,39 @@ def test_trace_runner_command_line(tmp_path):
     close(rd(0), wa[[0, 11]], 2e-4)
     close(rd(1), wb[[8]], 2e-4)
     close(rd(2), wa[[20, 13]], 2e-4)
+
+
+def test_served_through_the_llm_worker(tmp_path):
+    """The gRPC LLM worker loads a Vugotar checkpoint directory like any other model and streams a completion whose
+    tokens are the oracle's greedy continuation (byte-level tokenizer: one token per prompt byte after BOS)."""
+    from localai_tfp_amd.grpc import pb
+    from localai_tfp_amd.grpc.client import BackendClient
+    from localai_tfp_amd.grpc.server import AioServer
+    from localai_tfp_amd.workers.llm import LLMServicer
+    cfg = VU.make_config(**dict(SHAPES["plain"], vocab=300))
+    get = VU.synthetic_source(cfg, 12)
+    VU.save_checkpoint(cfg, get, str(tmp_path))
+    svc = LLMServicer(device="cpu")
+    server = AioServer(svc, "127.0.0.1:0", max_workers=4)
+    c = BackendClient(f"127.0.0.1:{server.port}")
+    try:
+        r = c.load_model(pb.ModelOptions(Model=str(tmp_path), ContextSize=256))
+        assert r.success, r.message
+        assert isinstance(svc.engine.model, VU.VugotarModel)
+        o = pb.PredictOptions(Prompt="hybrid", Tokens=6, Temperature=0.0, IgnoreEOS=True)
+        a = c.predict(o)
+        chunks = list(c.predict_stream(o))
+        assert a.tokens == 6 and b"".join(x.message for x in chunks) == a.message
+        tok = svc.engine.tok
+        seq = list(tok.encode("hybrid"))
+        assert a.prompt_tokens == len(seq)
+        tensors = {k: get(k) for k in get.names}
+        want = []
+        for _ in range(6):
+            want.append(int(oracle(cfg, tensors, seq + want)[-1].argmax()))
+        assert tok.decode(want).encode(errors="replace") == a.message or a.message == tok.decode(want).encode()
+    finally:
+        c.close()
+        if svc.engine is not None:
+            svc.engine.shutdown()
+        server.stop()
