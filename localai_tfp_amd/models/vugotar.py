@@ -190,8 +190,8 @@ class VugotarConfig:
             elif f.get("kind") == "moe":
                 r = f["router"]
                 sh = f.get("shared")
-                mlp = MlpCfg("moe", int(f["expert"]["ff"]), int(r["experts"]), int(r["top"]), float(r.get("scale", 1.0)),
-                             int(sh["ff"]) if sh else None)
+                mlp = MlpCfg("moe", int(f["expert"]["ff"]), int(r["experts"]), int(r["top"]),
+                             float(r.get("scale", 1.0)), int(sh["ff"]) if sh else None)
                 _need(0 < mlp.top <= mlp.experts, f"layer {i}: 1 <= top <= experts")
             else:
                 raise ValueError(f"layer {i}: unknown feed-forward {f.get('kind')!r}")
@@ -621,7 +621,8 @@ def tensor_shapes(cfg: VugotarConfig) -> dict:
                       p + "right.k": (r.kv_heads * r.dim, C), p + "right.k.conv": (r.kv_heads * r.dim, r.conv),
                       p + "right.v": (r.heads * r.vdim, C), p + "right.v.conv": (r.heads * r.vdim, r.conv),
                       p + "right.b": (r.heads, C), p + "right.a": (r.heads, C), p + "right.A_log": (r.heads,),
-                      p + "right.dt_bias": (r.heads,), p + "right.norm": (r.vdim,), p + "right.g": (r.heads * r.vdim, C),
+                      p + "right.dt_bias": (r.heads,), p + "right.norm": (r.vdim,),
+                      p + "right.g": (r.heads * r.vdim, C),
                       p + "right.o": (C, r.heads * r.vdim)})
         else:
             cc = m.inner + 2 * m.groups * m.state

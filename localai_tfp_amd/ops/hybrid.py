@@ -10,7 +10,8 @@
 * `causal_conv`: a per-channel causal convolution over time (optional bias and SiLU) whose last taps-1 inputs are
   carried per sequence;
 * `unit_norm_heads`, `scan_coefs`, `state_scan`: the pieces of a linear recurrence S <- a S + k u^T, o = S^T q per
-  head (S is [N, P], fp32, one per sequence and head, stored column-major). With `delta` the written value is u = c (v - S^T k) after
+  head (S is [N, P], fp32, one per sequence and head, stored column-major). With `delta` the written value is
+  u = c (v - S^T k) after
   the decay (gated delta rule), otherwise u = c v with an optional skip D v on the output (state-space duality form);
 * `gated_group_norm`: unit-RMS norm over groups of columns, a weight, and a SiLU gate before or after the norm;
 * `glu`: silu(a + bias) * (b + bias) with an optional per-row, per-column-group factor (routing weights of experts
@@ -276,7 +277,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
         mfma = mfma_ok
         big = MFMA_MIN_ROWS if mfma else GEMM_MIN_ROWS
         if lens is None or max(lens) < big or (not mfma and 0 < chunk < GEMM_MIN_ROWS):
-            rows_kernel(0, T - nd)  # (chunks shorter than a block of rows: a row's few visible keys suit the row kernel)
+            rows_kernel(0, T - nd)  # (mask chunks shorter than a block of rows: few visible keys, the row kernel's case)
             return out
         r, run0 = 0, None  # run0: first row of a run of consecutive short chunks
         for k, n in enumerate(lens):

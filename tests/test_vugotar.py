@@ -471,7 +471,8 @@ def test_unequal_batches_reuse_blocks_and_slots(dev, dt, tol):
         assert at[k] == len(reqs[k])
         close(torch.cat(got[k]), want[k], tol / 2 if dt == "bfloat16" else tol, dt == "bfloat16")
         # and the same request alone, in the same number format: no router tie falls differently here
-        close(torch.cat(got[k]), run_cuts(eng, "alone-" + k, reqs[k], [len(reqs[k])]), 2e-4 if dt == "float32" else 4e-3)
+        alone = run_cuts(eng, "alone-" + k, reqs[k], [len(reqs[k])])
+        close(torch.cat(got[k]), alone, 2e-4 if dt == "float32" else 4e-3)
     assert eng.bm.num_free == eng.bm.num_blocks - 1 and len(eng.state_slots.free) == 3
 
 
